@@ -1,0 +1,82 @@
+"""ctypes binding of libfgc_hip.so (the C ABI declared in include/fgc_hip.h).
+
+There is no fallback: if the shared library is missing, or a tensor is not on
+a HIP device, the call raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libfgc_hip.so")
+_lib = None
+
+c_i64p = ctypes.POINTER(ctypes.c_int64)
+_vp, _i32, _i64, _f32, _sz = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_size_t
+
+# name -> (restype, argtypes); must list every symbol of include/fgc_hip.h
+SIGNATURES = {
+    "fgc_version": (ctypes.c_int, []),
+    "fgc_error_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "fgc_bin_geometry_workspace_bytes": (_sz, [_i64]),
+    "fgc_bin_geometry_f32": (ctypes.c_int, [_vp, _i64, _i32, _i32, _i32, c_i64p, _i32, _f32, _i32, _vp, _vp,
+                                            _vp, _sz, _vp]),
+    "fgc_bin_points_f32": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, _i32, c_i64p, _vp, _vp, _vp, _vp, _vp]),
+    "fgc_binned_select_knn_workspace_bytes": (_sz, [_i64, _i32, _i32, c_i64p, _i32, _i32]),
+    "fgc_binned_select_knn_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, c_i64p, _i32, _i32, _i32, c_i64p, _vp,
+                                                 _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "fgc_index_replacer_i64": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
+    "fgc_binned_select_knn_grad_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp, _vp]),
+    "fgc_select_with_default_f32": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i32, _i32, _i64, _f32, _vp]),
+    "fgc_gravnet_aggregate_fwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp]),
+    "fgc_gravnet_aggregate_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32,
+                                                     _vp]),
+}
+
+ST_NONFINITE, ST_CLAMPED, ST_BAD_RANGE, ST_BAD_INDEX = 1, 2, 4, 8
+
+
+def lib():
+    """Load libfgc_hip.so once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "fastgraphcompute_amd: %s is missing - build it with "
+                "`python fastgraphcompute_amd/csrc/build.py` (hipcc, gfx950); there is no CPU fallback" % LIB_PATH)
+        l = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        msg = lib().fgc_error_string(rc).decode()
+        if rc == -3:
+            raise ValueError(msg)
+        raise RuntimeError("fastgraphcompute_amd: %s (code %d)" % (msg, rc))
+
+
+def require_device(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("fastgraphcompute_amd runs on MI355X (HIP) tensors only; got a %s tensor and "
+                               "there is no CPU fallback" % t.device)
+
+
+def stream_ptr():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def host_i64(values):
+    arr = (ctypes.c_int64 * len(values))(*[int(v) for v in values])
+    return arr

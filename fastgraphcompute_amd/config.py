@@ -1,0 +1,10 @@
+"""Run-time switches of the host wrappers."""
+
+# Read the device status word after each kNN call and raise on non-finite input
+# (one host synchronisation per call, as the reference's own checks do).  Set to
+# False inside latency-critical loops that validate their inputs elsewhere.
+sync_checks = True
+
+# Accumulate the kNN kernel's counters (distance evaluations, candidate chunks,
+# list insertions) into binned_select_knn.last_stats; used by the benchmark.
+collect_stats = False

@@ -1,0 +1,45 @@
+"""Compile libfgc_hip.so for gfx950 with hipcc (no torch headers involved).
+
+    python fastgraphcompute_amd/csrc/build.py
+
+-ffp-contract=off keeps every float operation a single IEEE operation (bin
+indices and squared distances are bit-identical to a sequential float32
+evaluation); packed-FP32 instruction selection is switched off.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SOURCES = ["fgc_binning.hip", "fgc_knn.hip", "fgc_ops.hip", "fgc_api.hip"]
+OUT = os.path.join(os.path.dirname(HERE), "libfgc_hip.so")
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+         "-Wno-unknown-warning-option"]
+
+
+def build(verbose=True, extra=()):
+    objs = []
+    procs = []
+    for src in SOURCES:
+        obj = os.path.join(HERE, src.replace(".hip", ".o"))
+        cmd = ["hipcc"] + FLAGS + list(extra) + ["-c", os.path.join(HERE, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((subprocess.Popen(cmd), src))
+        objs.append(obj)
+    for p, src in procs:
+        if p.wait() != 0:
+            raise RuntimeError("hipcc failed on " + src)
+    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT] + objs
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    for o in objs:
+        os.remove(o)
+    return OUT
+
+
+if __name__ == "__main__":
+    build(extra=sys.argv[1:])
+    print("built", OUT)

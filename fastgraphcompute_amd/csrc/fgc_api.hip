@@ -1,0 +1,117 @@
+// Whole-call entry points and bookkeeping of libfgc_hip.so.
+#include "fgc_common.h"
+#include "fgc_internal.h"
+
+extern "C" int fgc_version(void) { return 100; }
+
+extern "C" const char *fgc_error_string(int code)
+{
+    switch (code) {
+    case FGC_OK: return "success";
+    case FGC_EINVAL: return "invalid argument (shape, size or row splits)";
+    case FGC_ENOSPACE: return "workspace too small";
+    case FGC_EUNSUPPORTED: return "Unsupported number of binning dimensions.";
+    default: break;
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "unknown error";
+}
+
+namespace {
+struct KnnWorkspace {
+    size_t geom, partial, keys, vals, sort, bb, sc, sdir, total;
+    int ldc;
+};
+
+int64_t total_bins(int n_bin_dims, const int64_t *n_bins, int n_rs)
+{
+    int64_t b = n_rs - 1;
+    for (int d = 0; d < n_bin_dims; d++) {
+        if (n_bins[d] < 1 || n_bins[d] > (1ll << 31)) return -1;
+        if (b > (1ll << 31) / n_bins[d]) return -1;
+        b *= n_bins[d];
+    }
+    return b;
+}
+
+KnnWorkspace plan(int64_t n, int D, int nbd, const int64_t *n_bins, int n_rs, bool with_dir)
+{
+    KnnWorkspace w;
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off += fgc_align(bytes); return o; };
+    int64_t B = total_bins(nbd, n_bins, n_rs);
+    if (B < 0) B = 0;
+    w.ldc = (int)((n + 63) & ~63ll);
+    w.geom = take(FGC_GEOM_FLOATS * sizeof(float));
+    w.partial = take(fgc_bin_geometry_workspace_bytes(n));
+    w.keys = take((size_t)n * 4);
+    w.vals = take((size_t)n * 4);
+    w.sort = take(fgc_sort_workspace_bytes(n));
+    w.bb = take((size_t)(B + 1) * 4);
+    w.sc = take((size_t)w.ldc * D * 4);
+    w.sdir = take(with_dir ? (size_t)n : 0);
+    w.total = off;
+    return w;
+}
+}  // namespace
+
+extern "C" size_t fgc_binned_select_knn_workspace_bytes(int64_t n_vert, int32_t n_coords, int32_t n_bin_dims,
+                                                        const int64_t *n_bins, int32_t n_rs, int32_t K)
+{
+    (void)K;
+    if (n_vert <= 0 || !n_bins || n_bin_dims < 1 || n_bin_dims > FGC_MAX_BIN_DIMS) return 256;
+    return plan(n_vert, n_coords, n_bin_dims, n_bins, n_rs, true).total;
+}
+
+extern "C" int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
+                                         const int64_t *d_row_splits, const int64_t *row_splits_host,
+                                         int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
+                                         const int64_t *d_direction, int32_t tf_compat, int64_t *d_idx,
+                                         float *d_distsq, int32_t *d_status, uint64_t *d_stats, void *d_ws,
+                                         size_t ws_bytes, void *stream)
+{
+    if (n_vert < 0 || n_coords < 1 || n_rs < 2 || !row_splits_host || !n_bins) return FGC_EINVAL;
+    if (K < 1 || K > FGC_MAX_K) return FGC_EINVAL;
+    if (n_bin_dims < 2 || n_bin_dims > FGC_MAX_BIN_DIMS || n_bin_dims > n_coords) return FGC_EUNSUPPORTED;
+    if (n_vert >= (1ll << 31) - 64) return FGC_EINVAL;
+    // "Bin boundaries do not match row splits" of the reference, checked up front
+    if (row_splits_host[0] != 0 || row_splits_host[n_rs - 1] != n_vert) return FGC_EINVAL;
+    for (int r = 1; r < n_rs; r++)
+        if (row_splits_host[r] < row_splits_host[r - 1]) return FGC_EINVAL;
+    if (n_vert == 0) return FGC_OK;
+    if (!d_coords || !d_row_splits || !d_idx || !d_distsq || !d_ws) return FGC_EINVAL;
+    const int64_t B = total_bins(n_bin_dims, n_bins, n_rs);
+    if (B < 0 || B >= (1ll << 31)) return FGC_EINVAL;
+    const KnnWorkspace w = plan(n_vert, n_coords, n_bin_dims, n_bins, n_rs, d_direction != nullptr);
+    if (ws_bytes < w.total) return FGC_ENOSPACE;
+
+    hipStream_t s = (hipStream_t)stream;
+    char *ws = (char *)d_ws;
+    float *geom = (float *)(ws + w.geom);
+    uint32_t *keys = (uint32_t *)(ws + w.keys), *vals = (uint32_t *)(ws + w.vals);
+    int *bb = (int *)(ws + w.bb);
+    float *sc = (float *)(ws + w.sc);
+    unsigned char *sdir = d_direction ? (unsigned char *)(ws + w.sdir) : nullptr;
+
+    int rc = fgc_bin_geometry_f32(d_coords, n_vert, n_coords, n_bin_dims, 0, n_bins, 1, 0.f, 0, geom, d_status,
+                                  ws + w.partial, fgc_bin_geometry_workspace_bytes(n_vert), stream);
+    if (rc) return rc;
+    rc = fgc_launch_bin_keys(d_coords, (int)n_vert, n_coords, n_bin_dims, geom, d_row_splits, n_rs, keys,
+                             d_status, s);
+    if (rc) return rc;
+    int key_bits = 1;
+    while ((1ll << key_bits) < B) key_bits++;
+    uint32_t *skeys = nullptr, *order = nullptr;
+    rc = fgc_sort_keys(keys, vals, n_vert, key_bits, ws + w.sort, s, &skeys, &order);
+    if (rc) return rc;
+    rc = fgc_launch_bin_boundaries(skeys, (int)n_vert, (int)B, bb, s);
+    if (rc) return rc;
+    rc = fgc_launch_gather_sorted(d_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir, s);
+    if (rc) return rc;
+
+    KnnArgs a;
+    a.sc = sc; a.ldc = w.ldc; a.skeys = skeys; a.order = order; a.bb = bb; a.geom = geom; a.sdir = sdir;
+    a.n = (int)n_vert; a.D = n_coords; a.nbd = n_bin_dims; a.K = K; a.tf_compat = tf_compat;
+    a.out_idx = d_idx; a.out_dist = d_distsq; a.stats = (unsigned long long *)d_stats;
+    return fgc_launch_knn(a, s);
+}

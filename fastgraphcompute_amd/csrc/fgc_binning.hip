@@ -1,0 +1,515 @@
+// Binning geometry, per-point binning, and the stable LSD radix sort that puts
+// points into bin order (keys = flat bin index, 8-bit digits, LDS histograms,
+// wave-ballot ranking).  gfx950, wave64.
+#include "fgc_common.h"
+#include "fgc_internal.h"
+
+// ---------------------------------------------------------------------------
+// small utilities
+// ---------------------------------------------------------------------------
+__global__ void k_fill_u32(uint32_t *p, uint32_t v, int64_t n)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) p[i] = v;
+}
+
+int fgc_fill_u32(void *d, uint32_t v, int64_t n_words, hipStream_t s)
+{
+    if (n_words <= 0) return FGC_OK;
+    int64_t blocks = fgc_cdiv(n_words, 256 * 8);
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)blocks), dim3(256), 0, s, (uint32_t *)d, v, n_words);
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
+}
+
+__device__ __forceinline__ float wave_min_f(float v)
+{
+    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_max_f(float v)
+{
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// ---------------------------------------------------------------------------
+// geometry: per-dimension min / max of the binned coordinates
+// ---------------------------------------------------------------------------
+#define RANGE_BLOCKS_MAX 1024
+
+// partial[blk][0..4] = min, [5..9] = max, [10] = non-finite seen (as float 0/1)
+__global__ __launch_bounds__(256) void k_range_partial(const float *__restrict__ coords, int64_t n,
+                                                       int ld, int nbd, float *__restrict__ partial)
+{
+    float mn[FGC_MAX_BIN_DIMS], mx[FGC_MAX_BIN_DIMS];
+    int bad = 0;
+#pragma unroll
+    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) { mn[d] = INFINITY; mx[d] = -INFINITY; }
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+#pragma unroll
+        for (int d = 0; d < FGC_MAX_BIN_DIMS; d++)
+            if (d < nbd) {
+                float x = coords[i * ld + d];
+                bad |= !isfinite(x);
+                mn[d] = fminf(mn[d], x);
+                mx[d] = fmaxf(mx[d], x);
+            }
+    }
+    __shared__ float s_red[4][11];
+    const int lane = fgc_lane(), wv = threadIdx.x >> 6;
+#pragma unroll
+    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
+        float a = wave_min_f(mn[d]), b = wave_max_f(mx[d]);
+        if (lane == 0) { s_red[wv][d] = a; s_red[wv][5 + d] = b; }
+    }
+    unsigned long long anybad = fgc_ballot(bad != 0);
+    if (lane == 0) s_red[wv][10] = anybad ? 1.f : 0.f;
+    __syncthreads();
+    if (threadIdx.x < 11) {
+        int t = threadIdx.x;
+        float v = s_red[0][t];
+        for (int w = 1; w < 4; w++) {
+            float o = s_red[w][t];
+            v = (t < 5) ? fminf(v, o) : fmaxf(v, o);
+        }
+        partial[blockIdx.x * 11 + t] = v;
+    }
+}
+
+// One wave: reduce the partials and derive the geometry record.  Arithmetic
+// order as the reference's tensor ops: (max - min), +1 where the range is
+// zero, +1e-3, width = max_d(range_d / n_bins_d)  [or n_bins from a width].
+__global__ __launch_bounds__(64) void k_geometry(const float *__restrict__ partial, int nblk, int nbd,
+                                                 int mode, int nb_given, float bw_in, int pre_norm,
+                                                 int nb0, int nb1, int nb2, int nb3, int nb4,
+                                                 float *__restrict__ geom, int *__restrict__ status)
+{
+    const int lane = fgc_lane();
+    float mn[FGC_MAX_BIN_DIMS], mx[FGC_MAX_BIN_DIMS];
+    float bad = 0.f;
+#pragma unroll
+    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) { mn[d] = INFINITY; mx[d] = -INFINITY; }
+    for (int b = lane; b < nblk; b += 64) {
+#pragma unroll
+        for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
+            mn[d] = fminf(mn[d], partial[b * 11 + d]);
+            mx[d] = fmaxf(mx[d], partial[b * 11 + 5 + d]);
+        }
+        bad = fmaxf(bad, partial[b * 11 + 10]);
+    }
+#pragma unroll
+    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) { mn[d] = wave_min_f(mn[d]); mx[d] = wave_max_f(mx[d]); }
+    bad = wave_max_f(bad);
+    if (lane != 0) return;
+    const int nb_in[FGC_MAX_BIN_DIMS] = {nb0, nb1, nb2, nb3, nb4};
+    int flags = bad > 0.f ? FGC_ST_NONFINITE : 0;
+    float rng[FGC_MAX_BIN_DIMS];
+    float bw = bw_in;
+    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
+        if (d >= nbd) { geom[FGC_GEOM_MIN + d] = 0.f; continue; }
+        float sub = pre_norm ? 0.f : mn[d];
+        float lo = pre_norm ? mn[d] : (mn[d] - sub);
+        float hi = pre_norm ? mx[d] : (mx[d] - sub);
+        if (lo == hi) hi = hi + 1.0f;
+        hi = hi + 1e-3f;
+        if (!isfinite(hi)) hi = 1.0f;
+        if (!(hi > 0.f)) flags |= FGC_ST_BAD_RANGE;
+        rng[d] = hi;
+        geom[FGC_GEOM_MIN + d] = sub;
+    }
+    int nbo[FGC_MAX_BIN_DIMS] = {1, 1, 1, 1, 1};
+    if (mode == 0) {
+        float w = -INFINITY;
+        for (int d = 0; d < nbd; d++) {
+            nbo[d] = nb_in[d];
+            w = fmaxf(w, rng[d] / (float)nb_in[d]);
+        }
+        bw = w;
+    } else {
+        for (int d = 0; d < nbd; d++)
+            nbo[d] = nb_given ? nb_in[d] : (int)(long long)(rng[d] / bw) + 1;
+    }
+    for (int d = 0; d < nbd; d++)
+        if (nbo[d] <= 0) flags |= FGC_ST_BAD_RANGE;
+    if (!(bw > 0.f)) flags |= FGC_ST_BAD_RANGE;
+    geom[FGC_GEOM_BW] = bw;
+    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) geom[FGC_GEOM_NB + d] = __int_as_float(nbo[d]);
+    geom[FGC_GEOM_FLAGS] = __int_as_float(flags);
+    for (int d = 12; d < FGC_GEOM_FLOATS; d++) geom[d] = 0.f;
+    if (status && flags) atomicOr(&status[0], flags);
+}
+
+extern "C" size_t fgc_bin_geometry_workspace_bytes(int64_t n_vert)
+{
+    (void)n_vert;
+    return fgc_align((size_t)RANGE_BLOCKS_MAX * 11 * sizeof(float));
+}
+
+extern "C" int fgc_bin_geometry_f32(const float *d_coords, int64_t n_vert, int32_t ld_coords,
+                                    int32_t n_bin_dims, int32_t mode, const int64_t *n_bins_in,
+                                    int32_t n_bins_given, float bin_width_in, int32_t pre_normalized,
+                                    float *d_geom, int32_t *d_status, void *d_ws, size_t ws_bytes,
+                                    void *stream)
+{
+    if (n_vert <= 0 || n_bin_dims < 1 || n_bin_dims > FGC_MAX_BIN_DIMS || ld_coords < n_bin_dims)
+        return FGC_EINVAL;
+    if (!d_coords || !d_geom || !d_ws) return FGC_EINVAL;
+    if (ws_bytes < fgc_bin_geometry_workspace_bytes(n_vert)) return FGC_ENOSPACE;
+    if (mode == 0 && (!n_bins_in || !n_bins_given)) return FGC_EINVAL;
+    int nb[FGC_MAX_BIN_DIMS] = {1, 1, 1, 1, 1};
+    if (n_bins_in && n_bins_given)
+        for (int d = 0; d < n_bin_dims; d++) {
+            if (n_bins_in[d] > 0x7fffffff) return FGC_EINVAL;
+            nb[d] = (int)n_bins_in[d];
+        }
+    hipStream_t s = (hipStream_t)stream;
+    int nblk = (int)fgc_cdiv(n_vert, 256 * 4);
+    if (nblk > RANGE_BLOCKS_MAX) nblk = RANGE_BLOCKS_MAX;
+    hipLaunchKernelGGL(k_range_partial, dim3(nblk), dim3(256), 0, s, d_coords, n_vert, (int)ld_coords,
+                       (int)n_bin_dims, (float *)d_ws);
+    FGC_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_geometry, dim3(1), dim3(64), 0, s, (const float *)d_ws, nblk, (int)n_bin_dims,
+                       (int)mode, (int)n_bins_given, bin_width_in, (int)pre_normalized, nb[0], nb[1],
+                       nb[2], nb[3], nb[4], d_geom, d_status);
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
+}
+
+// ---------------------------------------------------------------------------
+// per-point binning
+// ---------------------------------------------------------------------------
+struct BinGeom {
+    float mn[FGC_MAX_BIN_DIMS];
+    float bw;
+    int nb[FGC_MAX_BIN_DIMS];
+};
+
+__device__ __forceinline__ BinGeom load_geom(const float *__restrict__ geom)
+{
+    BinGeom g;
+#pragma unroll
+    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
+        g.mn[d] = geom[FGC_GEOM_MIN + d];
+        g.nb[d] = __float_as_int(geom[FGC_GEOM_NB + d]);
+    }
+    g.bw = geom[FGC_GEOM_BW];
+    return g;
+}
+
+// number of row-split entries rs[1..n_rs-1] that are <= v  (the event of point v)
+__device__ __forceinline__ int event_of(const int64_t *__restrict__ rs, int n_rs, int64_t v)
+{
+    int lo = 1, hi = n_rs;  // first r in [1, n_rs) with rs[r] > v
+    while (lo < hi) {
+        int mid = (lo + hi) >> 1;
+        if (rs[mid] > v) hi = mid; else lo = mid + 1;
+    }
+    return lo - 1;
+}
+
+// bin index of one coordinate: floorf((x - min) / bw + 1e-3f), clamped
+__device__ __forceinline__ int bin_of(float x, float mn, float bw, int nb, int &clamped)
+{
+    float q = (x - mn) / bw;
+    long long b = (long long)floorf(q + 1e-3f);
+    if (b < 0) { b = 0; clamped = 1; }
+    else if (b >= nb) { b = nb - 1; clamped = 1; }
+    return (int)b;
+}
+
+__global__ __launch_bounds__(256) void k_bin_points(const float *__restrict__ coords, int64_t n, int ld,
+                                                    int nbd, const float *__restrict__ geom,
+                                                    const int64_t *__restrict__ rs, int n_rs,
+                                                    int64_t n_total_bins,
+                                                    int64_t *__restrict__ assigned,
+                                                    int64_t *__restrict__ flat,
+                                                    unsigned long long *__restrict__ n_per_bin,
+                                                    int *__restrict__ status)
+{
+    int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (v >= n) return;
+    BinGeom g = load_geom(geom);
+    int clamped = 0;
+    int64_t f = 0, stride = 1;
+    int b[FGC_MAX_BIN_DIMS];
+#pragma unroll
+    for (int d = FGC_MAX_BIN_DIMS - 1; d >= 0; d--)
+        if (d < nbd) {
+            b[d] = bin_of(coords[v * ld + d], g.mn[d], g.bw, g.nb[d], clamped);
+            f += (int64_t)b[d] * stride;
+            stride *= g.nb[d];
+        }
+    int ev = event_of(rs, n_rs, v);
+    f += (int64_t)ev * stride;
+    if (clamped && status) atomicOr(&status[0], FGC_ST_CLAMPED);
+    if (assigned) {
+#pragma unroll
+        for (int d = 0; d < FGC_MAX_BIN_DIMS; d++)
+            if (d < nbd) assigned[v * (nbd + 1) + 1 + d] = b[d];
+    }
+    if (f >= n_total_bins) return;  // point beyond the last row split: left out, as the reference does
+    if (assigned) assigned[v * (nbd + 1)] = ev;
+    if (flat) flat[v] = f;
+    if (n_per_bin) atomicAdd(&n_per_bin[f], 1ull);
+}
+
+extern "C" int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t ld_coords,
+                                  int32_t n_bin_dims, const float *d_geom, const int64_t *d_row_splits,
+                                  int32_t n_rs, const int64_t *n_bins_host, int64_t *d_assigned,
+                                  int64_t *d_flat, int64_t *d_n_per_bin, int32_t *d_status, void *stream)
+{
+    if (n_vert < 0 || n_bin_dims < 1 || n_bin_dims > FGC_MAX_BIN_DIMS || n_rs < 2 || !n_bins_host)
+        return FGC_EINVAL;
+    if (n_vert == 0) return FGC_OK;
+    int64_t total = n_rs - 1;
+    for (int d = 0; d < n_bin_dims; d++) {
+        if (n_bins_host[d] <= 0) return FGC_EINVAL;
+        if (total > INT64_MAX / n_bins_host[d]) return FGC_EINVAL;
+        total *= n_bins_host[d];
+    }
+    hipStream_t s = (hipStream_t)stream;
+    hipLaunchKernelGGL(k_bin_points, dim3((unsigned)fgc_cdiv(n_vert, 256)), dim3(256), 0, s, d_coords,
+                       n_vert, (int)ld_coords, (int)n_bin_dims, d_geom, d_row_splits, (int)n_rs, total,
+                       d_assigned, d_flat, (unsigned long long *)d_n_per_bin, d_status);
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
+}
+
+// ---------------------------------------------------------------------------
+// sort keys for the kNN pipeline: key = flat bin (uint32)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_bin_keys(const float *__restrict__ coords, int n, int ld, int nbd,
+                                                  const float *__restrict__ geom,
+                                                  const int64_t *__restrict__ rs, int n_rs,
+                                                  uint32_t *__restrict__ keys, int *__restrict__ status)
+{
+    int v = blockIdx.x * blockDim.x + threadIdx.x;
+    if (v >= n) return;
+    BinGeom g = load_geom(geom);
+    int clamped = 0;
+    uint32_t f = 0, stride = 1;
+#pragma unroll
+    for (int d = FGC_MAX_BIN_DIMS - 1; d >= 0; d--)
+        if (d < nbd) {
+            int b = bin_of(coords[(int64_t)v * ld + d], g.mn[d], g.bw, g.nb[d], clamped);
+            f += (uint32_t)b * stride;
+            stride *= (uint32_t)g.nb[d];
+        }
+    f += (uint32_t)event_of(rs, n_rs, v) * stride;
+    if (clamped && status) atomicOr(&status[0], FGC_ST_CLAMPED);
+    keys[v] = f;
+}
+
+// ---------------------------------------------------------------------------
+// LSD radix sort, 8-bit digits, stable.  Tile = 4 waves x 16 chunks x 64 keys.
+// ---------------------------------------------------------------------------
+#define RS_TILE 4096
+#define RS_CHUNKS 16
+
+// lanes of this wave holding the same digit (valid lanes only)
+__device__ __forceinline__ unsigned long long match_digit(int digit, bool valid)
+{
+    unsigned long long m = fgc_ballot(valid);
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+        unsigned long long s = fgc_ballot(valid && ((digit >> b) & 1));
+        m &= ((digit >> b) & 1) ? s : ~s;
+    }
+    return m;
+}
+
+// block_hist is digit-major: block_hist[digit * nblk + blk]
+__global__ __launch_bounds__(256) void k_rs_hist(const uint32_t *__restrict__ keys, int n, int shift,
+                                                 int nblk, uint32_t *__restrict__ block_hist)
+{
+    __shared__ uint32_t s_h[256];
+    s_h[threadIdx.x] = 0;
+    __syncthreads();
+    const int base = blockIdx.x * RS_TILE;
+#pragma unroll 4
+    for (int c = 0; c < RS_CHUNKS; c++) {
+        int i = base + c * 256 + threadIdx.x;
+        if (i < n) atomicAdd(&s_h[(keys[i] >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    block_hist[threadIdx.x * nblk + blockIdx.x] = s_h[threadIdx.x];
+}
+
+// in-place exclusive scan of `len` uint32 values by one 1024-thread block;
+// if total != NULL it receives the sum
+__global__ __launch_bounds__(1024) void k_scan_excl_u32(uint32_t *__restrict__ a, int len,
+                                                        uint32_t *__restrict__ total)
+{
+    __shared__ uint32_t s_w[16];
+    const int t = threadIdx.x, lane = t & 63, wv = t >> 6;
+    const int per = (len + 1023) / 1024;
+    const int lo = min(len, t * per), hi = min(len, lo + per);
+    uint32_t sum = 0;
+    for (int i = lo; i < hi; i++) sum += a[i];
+    uint32_t incl = sum;
+    for (int o = 1; o < 64; o <<= 1) {
+        uint32_t u = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += u;
+    }
+    if (lane == 63) s_w[wv] = incl;
+    __syncthreads();
+    uint32_t woff = 0;
+    for (int w = 0; w < wv; w++) woff += s_w[w];
+    uint32_t run = woff + incl - sum;
+    for (int i = lo; i < hi; i++) {
+        uint32_t v = a[i];
+        a[i] = run;
+        run += v;
+    }
+    if (total && t == 1023) *total = run;
+}
+
+__global__ __launch_bounds__(256) void k_rs_scatter(const uint32_t *__restrict__ keys_in,
+                                                    const uint32_t *__restrict__ vals_in,
+                                                    uint32_t *__restrict__ keys_out,
+                                                    uint32_t *__restrict__ vals_out, int n, int shift,
+                                                    int nblk, const uint32_t *__restrict__ block_hist)
+{
+    __shared__ uint32_t s_cnt[4][256];
+    const int lane = fgc_lane(), wv = threadIdx.x >> 6;
+    volatile uint32_t *cnt = s_cnt[wv];
+    for (int i = lane; i < 256; i += 64) cnt[i] = 0;
+    const int base = blockIdx.x * RS_TILE + wv * (RS_TILE / 4);
+    uint32_t key[RS_CHUNKS];
+    // pass 1: per-wave digit counts
+#pragma unroll
+    for (int c = 0; c < RS_CHUNKS; c++) {
+        int i = base + c * 64 + lane;
+        bool valid = i < n;
+        key[c] = valid ? keys_in[i] : 0u;
+        int digit = (int)((key[c] >> shift) & 255u);
+        unsigned long long m = match_digit(digit, valid);
+        if (valid && fgc_mbcnt(m) == 0) cnt[digit] = cnt[digit] + (uint32_t)__popcll(m);
+    }
+    __syncthreads();
+    // per-digit exclusive offsets of the four waves on top of the global base
+    {
+        int t = threadIdx.x;
+        uint32_t g = block_hist[t * nblk + blockIdx.x];
+        for (int w = 0; w < 4; w++) {
+            uint32_t c = s_cnt[w][t];
+            s_cnt[w][t] = g;
+            g += c;
+        }
+    }
+    __syncthreads();
+    // pass 2: same order, running offsets -> stable
+#pragma unroll
+    for (int c = 0; c < RS_CHUNKS; c++) {
+        int i = base + c * 64 + lane;
+        bool valid = i < n;
+        int digit = (int)((key[c] >> shift) & 255u);
+        unsigned long long m = match_digit(digit, valid);
+        int rank = fgc_mbcnt(m);
+        uint32_t off = valid ? cnt[digit] : 0u;
+        if (valid && rank == 0) cnt[digit] = off + (uint32_t)__popcll(m);
+        if (valid) {
+            uint32_t pos = off + (uint32_t)rank;
+            keys_out[pos] = key[c];
+            vals_out[pos] = vals_in ? vals_in[i] : (uint32_t)i;
+        }
+    }
+}
+
+size_t fgc_sort_workspace_bytes(int64_t n)
+{
+    int64_t nblk = fgc_cdiv(n > 0 ? n : 1, RS_TILE);
+    return fgc_align((size_t)n * 4) * 2 /* ping-pong keys / vals */ + fgc_align((size_t)nblk * 256 * 4);
+}
+
+// Sorts (keys, identity) stably by the low `key_bits` bits.  On return
+// *keys_sorted / *vals_sorted point at the buffers holding the result
+// (either the caller's primary pair or the alternates inside the workspace).
+int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void *d_ws, hipStream_t s,
+                  uint32_t **keys_sorted, uint32_t **vals_sorted)
+{
+    if (n >= (1ll << 31)) return FGC_EINVAL;
+    char *w = (char *)d_ws;
+    uint32_t *k_alt = (uint32_t *)w; w += fgc_align((size_t)n * 4);
+    uint32_t *v_alt = (uint32_t *)w; w += fgc_align((size_t)n * 4);
+    uint32_t *hist = (uint32_t *)w;
+    int nblk = (int)fgc_cdiv(n, RS_TILE);
+    if ((int64_t)nblk * 256 >= (1ll << 31)) return FGC_EINVAL;
+    uint32_t *kin = keys, *vin = nullptr, *kout = k_alt, *vout = v_alt;
+    int passes = (key_bits + 7) / 8;
+    if (passes < 1) passes = 1;
+    for (int p = 0; p < passes; p++) {
+        int shift = p * 8;
+        hipLaunchKernelGGL(k_rs_hist, dim3(nblk), dim3(256), 0, s, kin, (int)n, shift, nblk, hist);
+        FGC_LAUNCH_CHECK();
+        hipLaunchKernelGGL(k_scan_excl_u32, dim3(1), dim3(1024), 0, s, hist, nblk * 256, (uint32_t *)nullptr);
+        FGC_LAUNCH_CHECK();
+        hipLaunchKernelGGL(k_rs_scatter, dim3(nblk), dim3(256), 0, s, kin, vin, kout, vout, (int)n, shift,
+                           nblk, hist);
+        FGC_LAUNCH_CHECK();
+        kin = kout; vin = vout;
+        if (kout == k_alt) { kout = keys; vout = vals; } else { kout = k_alt; vout = v_alt; }
+    }
+    *keys_sorted = kin;
+    *vals_sorted = vin;
+    return FGC_OK;
+}
+
+// bin_boundaries[b] = first sorted position whose key is >= b, for b in [0, n_bins_total]
+__global__ __launch_bounds__(256) void k_bin_boundaries(const uint32_t *__restrict__ skeys, int n,
+                                                        int n_bins_total, int *__restrict__ bb)
+{
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i > n) return;
+    long long prev = (i > 0) ? (long long)skeys[i - 1] : -1ll;
+    long long cur = (i < n) ? (long long)skeys[i] : (long long)n_bins_total;
+    if (cur > n_bins_total) cur = n_bins_total;
+    for (long long b = prev + 1; b <= cur; b++) bb[b] = i;
+}
+
+// sorted structure-of-arrays coordinates: sc[d * ldc + i] = coords[order[i]][d]
+__global__ __launch_bounds__(256) void k_gather_sorted(const float *__restrict__ coords,
+                                                       const uint32_t *__restrict__ order, int n, int D,
+                                                       int ldc, float *__restrict__ sc,
+                                                       const int64_t *__restrict__ direction,
+                                                       unsigned char *__restrict__ sdir)
+{
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint32_t o = order[i];
+    for (int d = 0; d < D; d++) sc[(int64_t)d * ldc + i] = coords[(int64_t)o * D + d];
+    if (sdir) {
+        int64_t v = direction[o];
+        sdir[i] = (unsigned char)((v >= 0 && v <= 2) ? v : 3);
+    }
+}
+
+int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, const float *d_geom,
+                        const int64_t *d_rs, int n_rs, uint32_t *d_keys, int *d_status, hipStream_t s)
+{
+    hipLaunchKernelGGL(k_bin_keys, dim3((unsigned)fgc_cdiv(n, 256)), dim3(256), 0, s, d_coords, n, ld, nbd,
+                       d_geom, d_rs, n_rs, d_keys, d_status);
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
+}
+
+int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int n_bins_total, int *bb, hipStream_t s)
+{
+    hipLaunchKernelGGL(k_bin_boundaries, dim3((unsigned)fgc_cdiv((int64_t)n + 1, 256)), dim3(256), 0, s, skeys,
+                       n, n_bins_total, bb);
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
+}
+
+int fgc_launch_gather_sorted(const float *coords, const uint32_t *order, int n, int D, int ldc, float *sc,
+                             const int64_t *direction, unsigned char *sdir, hipStream_t s)
+{
+    hipLaunchKernelGGL(k_gather_sorted, dim3((unsigned)fgc_cdiv(n, 256)), dim3(256), 0, s, coords, order, n,
+                       D, ldc, sc, direction, sdir);
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
+}

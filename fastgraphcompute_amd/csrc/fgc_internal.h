@@ -1,0 +1,32 @@
+// Launchers shared between the translation units of libfgc_hip.so.
+#pragma once
+#include "fgc_common.h"
+
+size_t fgc_sort_workspace_bytes(int64_t n);
+int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void *d_ws, hipStream_t s,
+                  uint32_t **keys_sorted, uint32_t **vals_sorted);
+int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, const float *d_geom,
+                        const int64_t *d_rs, int n_rs, uint32_t *d_keys, int *d_status, hipStream_t s);
+int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int n_bins_total, int *bb, hipStream_t s);
+int fgc_launch_gather_sorted(const float *coords, const uint32_t *order, int n, int D, int ldc, float *sc,
+                             const int64_t *direction, unsigned char *sdir, hipStream_t s);
+
+// kNN search over bin-sorted points (fgc_knn.hip)
+struct KnnArgs {
+    const float *sc;            // sorted coordinates, structure of arrays [D][ldc]
+    int ldc;
+    const uint32_t *skeys;      // sorted flat bin per point
+    const uint32_t *order;      // sorted position -> original row
+    const int *bb;              // bin boundaries [n_bins_total + 1]
+    const float *geom;          // geometry record
+    const unsigned char *sdir;  // sorted direction flags or NULL
+    int n;                      // points
+    int D;                      // coordinates per point
+    int nbd;                    // binned dimensions
+    int K;
+    int tf_compat;
+    int64_t *out_idx;           // [n, K] original order
+    float *out_dist;            // [n, K]
+    unsigned long long *stats;  // optional counters
+};
+int fgc_launch_knn(const KnnArgs &a, hipStream_t s);

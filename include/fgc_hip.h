@@ -1,0 +1,177 @@
+/*
+ * fgc_hip.h - C ABI of libfgc_hip.so, the MI355X (gfx950) implementation of
+ * FastGraphCompute's graph-building path.
+ *
+ * Conventions
+ *   - Every pointer named d_* is device memory on the current HIP device; the
+ *     caller owns all of it, including the workspace.  The library allocates
+ *     nothing and frees nothing.
+ *   - `stream` is a hipStream_t passed as void*.  All work is enqueued on it
+ *     and the call returns without synchronising; results are valid once the
+ *     stream has reached that point.
+ *   - Return value: 0 on success, a negative FGC_E* code for rejected
+ *     arguments, a positive hipError_t for a failed launch.  No C++ exception
+ *     crosses this boundary and the process is never exit()ed.
+ *   - d_status (where present) is an int32[FGC_STATUS_WORDS] device array the
+ *     kernels OR anomaly bits into (the reference printf()s from the kernel
+ *     instead); the caller reads it whenever it synchronises anyway.
+ *   - Citations name the reference interface each entry point replaces, as
+ *     fastgraphcompute/extensions/<file>:<line>.
+ */
+#ifndef FGC_HIP_H_
+#define FGC_HIP_H_
+
+#include <stdint.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FGC_OK 0
+#define FGC_EINVAL (-1)      /* bad shape / unsupported size                  */
+#define FGC_ENOSPACE (-2)    /* workspace too small                           */
+#define FGC_EUNSUPPORTED (-3)/* e.g. number of binned dims outside 1..5       */
+
+#define FGC_MAX_BIN_DIMS 5
+#define FGC_MAX_K 256        /* neighbours per query the kNN kernel supports  */
+#define FGC_STATUS_WORDS 4
+/* bits of d_status[0] */
+#define FGC_ST_NONFINITE 1   /* a binned coordinate is inf/nan                */
+#define FGC_ST_CLAMPED 2     /* a coordinate fell outside the grid (clamped)  */
+#define FGC_ST_BAD_RANGE 4   /* range / bin width / n_bins not positive       */
+#define FGC_ST_BAD_INDEX 8   /* neighbour index >= n_vert seen (gradient)     */
+
+/* Library version (major*100 + minor) and the text for a return code. */
+int fgc_version(void);
+const char *fgc_error_string(int code);
+
+/* ---------------------------------------------------------------------------
+ * Binning geometry.  Replaces the tensor preprocessing of bin_by_coordinates
+ * (bin_by_coordinates.cpp:57-111, same arithmetic as bin_by_coordinates.py:
+ * 40-92): global per-dimension minimum, range (+1 where zero, +1e-3), and
+ * either the cubic bin width max_d(range_d / n_bins_d) from given n_bins
+ * (mode 0) or n_bins_d = int(range_d / bin_width) + 1 from a given width
+ * (mode 1).  All in single float32 operations.
+ *
+ *   d_coords     [n_vert, ld_coords] float32, first n_bin_dims columns binned
+ *   d_geom       out, float32[FGC_GEOM_FLOATS]: min[5], bin_width, then the
+ *                n_bins[5] as int32 bit patterns and a flags word
+ *   n_bins_in    host array [n_bin_dims] (mode 0; mode 1 with given n_bins)
+ *   bin_width_in used when mode == 1
+ *   pre_normalized != 0: minimum taken as 0 (coordinates used as they are)
+ *   d_ws         workspace of fgc_bin_geometry_workspace_bytes(n_vert) bytes
+ */
+#define FGC_GEOM_FLOATS 16
+size_t fgc_bin_geometry_workspace_bytes(int64_t n_vert);
+int fgc_bin_geometry_f32(const float *d_coords, int64_t n_vert, int32_t ld_coords,
+                         int32_t n_bin_dims, int32_t mode, const int64_t *n_bins_in,
+                         int32_t n_bins_given, float bin_width_in, int32_t pre_normalized,
+                         float *d_geom, int32_t *d_status, void *d_ws, size_t ws_bytes,
+                         void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Per-point binning.  Replaces bin_by_coordinates_cuda_fn
+ * (bin_by_coordinates_cuda_kernel.cu:119-172; CPU twin
+ * bin_by_coordinates_cpu.cpp:7-99): bin of a coordinate =
+ * floorf((x - min) / bin_width + 1e-3f) clamped to [0, n_bins-1]; flat index
+ * row-major with dimension 0 most significant, plus event * prod(n_bins).
+ *
+ *   d_geom        as written by fgc_bin_geometry_f32
+ *   d_row_splits  int64 [n_rs]
+ *   d_assigned    out int64 [n_vert, n_bin_dims+1] (col 0 = event) or NULL
+ *   d_flat        out int64 [n_vert] or NULL
+ *   d_n_per_bin   out int64 [n_total_bins], must be zeroed by the caller, or NULL
+ */
+int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t ld_coords,
+                       int32_t n_bin_dims, const float *d_geom, const int64_t *d_row_splits,
+                       int32_t n_rs, const int64_t *n_bins_host, int64_t *d_assigned,
+                       int64_t *d_flat, int64_t *d_n_per_bin, int32_t *d_status, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Whole forward of binned_select_knn.  Replaces BinnedKNNAutograd::forward
+ * (binned_knn_autograd_kernel.cpp:85-209), i.e. bin_by_coordinates on the
+ * first n_bin_dims coordinates, the sort by flat bin, binned_select_knn_cuda_fn
+ * (binned_select_knn_cuda_kernel.cu:252-384), index_replacer_cuda_fn and the
+ * scatter back to the original order, in one call.
+ *
+ *   d_coords      [n_vert, n_coords] float32 row-major (original order)
+ *   d_row_splits  int64 [n_rs] on the device; row_splits_host the same values
+ *                 on the host (used to size the launch)
+ *   n_bins        host array [n_bin_dims], bins per binned dimension; the caller
+ *                 evaluates the reference's heuristic (calculate_optimal_bins,
+ *                 :67-82) or passes the user's n_bins
+ *   d_direction   int64 [n_vert] or NULL (0: only neighbour, 1: only query,
+ *                 2: neither; binned_select_knn_cuda_kernel.cu:120-122,194-196)
+ *   d_idx         out int64 [n_vert, K]: slot 0 the query itself, then its
+ *                 K-1 nearest points of the same event by increasing distance,
+ *                 -1 (or the query's index if tf_compat) where the event has
+ *                 fewer than K points
+ *   d_distsq      out float32 [n_vert, K], 0 for slot 0 and for padding
+ *   d_stats       optional uint64[4] device counters, accumulated: [0] distance
+ *                 evaluations, [1] candidate chunks visited, [2] insertions;
+ *                 NULL to skip
+ */
+size_t fgc_binned_select_knn_workspace_bytes(int64_t n_vert, int32_t n_coords,
+                                             int32_t n_bin_dims, const int64_t *n_bins,
+                                             int32_t n_rs, int32_t K);
+int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
+                              const int64_t *d_row_splits, const int64_t *row_splits_host,
+                              int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
+                              const int64_t *d_direction, int32_t tf_compat,
+                              int64_t *d_idx, float *d_distsq, int32_t *d_status,
+                              uint64_t *d_stats, void *d_ws, size_t ws_bytes, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Replaces index_replacer_cuda_fn (index_replacer_cuda_kernel.cu:30-59):
+ * out[i] = in[i] if in[i] < 0 or in[i] >= n_repl, else repl[in[i]].
+ */
+int fgc_index_replacer_i64(const int64_t *d_in, const int64_t *d_repl, int64_t *d_out,
+                           int64_t n, int64_t n_repl, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Replaces binned_select_knn_grad_cuda_fn
+ * (binned_select_knn_grad_cuda_kernel.cu:90-164; CPU twin
+ * binned_select_knn_grad_cpu.cpp:96-165):
+ *   g[i,c]      = -2 sum_k gd[i,k] (x[n_ik,c] - x[i,c])
+ *   g[n_ik,c]  +=  2 gd[i,k] (x[n_ik,c] - x[i,c])          (n_ik < 0 skipped)
+ * d_grad_coords [n_vert, n_coords] is fully overwritten.
+ */
+int fgc_binned_select_knn_grad_f32(const float *d_grad_distsq, const int64_t *d_idx,
+                                   const float *d_coords, float *d_grad_coords,
+                                   int64_t n_vert, int32_t K, int32_t n_coords,
+                                   int32_t *d_status, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Replaces select_with_default (oc_helper.py:232-271) for float32 features:
+ * out[v,k,:] = feat[idx[v,k],:], or default_value where idx[v,k] == -1.
+ */
+int fgc_select_with_default_f32(const int64_t *d_idx, const float *d_feat, float *d_out,
+                                int64_t n_vert, int32_t K, int32_t n_feat, int64_t n_feat_rows,
+                                float default_value, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * GravNet neighbour aggregation, fused.  Replaces the tensor ops of
+ * GravNetOp.forward, gnn_ops.py:90-102 (exp(-10 d^2) weights, gather with
+ * default 0, multiply, mean and max over the K slots) without materialising the
+ * [n_vert, K, P] tensor.
+ *   d_fmean, d_fmax  out float32 [n_vert, P]
+ *   d_argmax         out int32 [n_vert, P]: slot of the (first) maximum
+ * Backward: given d(loss)/d(fmean), d(loss)/d(fmax) it accumulates
+ *   d_grad_feat   [n_feat_rows, P], must be zeroed by the caller
+ *   d_grad_distsq [n_vert, K], fully overwritten
+ */
+int fgc_gravnet_aggregate_fwd_f32(const int64_t *d_idx, const float *d_distsq,
+                                  const float *d_feat, float *d_fmean, float *d_fmax,
+                                  int32_t *d_argmax, int64_t n_vert, int32_t K, int32_t P,
+                                  void *stream);
+int fgc_gravnet_aggregate_bwd_f32(const int64_t *d_idx, const float *d_distsq,
+                                  const float *d_feat, const int32_t *d_argmax,
+                                  const float *d_grad_fmean, const float *d_grad_fmax,
+                                  float *d_grad_feat, float *d_grad_distsq, int64_t n_vert,
+                                  int32_t K, int32_t P, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FGC_HIP_H_ */

@@ -1,0 +1,150 @@
+"""binned_select_knn on the GPU against the CPU checker and brute force."""
+import numpy as np
+import pytest
+import torch
+
+from tests.util import assert_knn_equal, check_knn_properties
+
+pytestmark = pytest.mark.gpu
+
+
+def _gpu_knn(K, coords, rs, **kw):
+    from fastgraphcompute_amd import binned_select_knn
+    for k in ("direction", "n_bins"):
+        if kw.get(k) is not None and not torch.is_tensor(kw[k]):
+            kw[k] = torch.as_tensor(kw[k], device="cuda")
+    idx, dist = binned_select_knn(K, torch.as_tensor(coords, device="cuda"),
+                                  torch.as_tensor(rs, device="cuda"), **kw)
+    assert idx.dtype == torch.int64 and dist.dtype == torch.float32
+    return idx.cpu().numpy(), dist.cpu().numpy()
+
+
+def _check(oracle, K, coords, rs, threads=8, **kw):
+    gi, gd = _gpu_knn(K, coords, rs, **kw)
+    okw = {k: (v.cpu().numpy() if torch.is_tensor(v) else v) for k, v in kw.items()}
+    oi, od = oracle.binned_select_knn(K, coords, rs, n_threads=threads, **okw)
+    assert_knn_equal(gi, gd, oi, od)
+    return gi, gd
+
+
+def test_cfg1_full(oracle):
+    from fastgraphcompute_amd.workloads import cfg1_uniform_small
+    w = cfg1_uniform_small()
+    gi, gd = _check(oracle, w["K"], w["coords"], w["row_splits"])
+    check_knn_properties(gi, gd, w["coords"], w["row_splits"], w["K"])
+    bi, bd = oracle.knn_brute(w["K"], w["coords"], w["row_splits"])
+    assert_knn_equal(gi, gd, bi, bd, "vs brute force")
+
+
+@pytest.mark.parametrize("name,scale", [("cfg2", 0.1), ("cfg4", 0.03), ("cfg5", 0.04)])
+def test_benchmark_shapes_scaled(oracle, name, scale):
+    from fastgraphcompute_amd.workloads import CONFIGS
+    w = CONFIGS[name](scale)
+    gi, gd = _check(oracle, w["K"], w["coords"], w["row_splits"])
+    check_knn_properties(gi, gd, w["coords"], w["row_splits"], w["K"])
+
+
+@pytest.mark.parametrize("D", [2, 3, 4, 5, 6, 7, 8, 9, 12])
+def test_dimensions(oracle, D):
+    rng = np.random.default_rng(40 + D)
+    coords = rng.random((3000, D)).astype(np.float32)
+    _check(oracle, 10, coords, [0, 1000, 1500, 3000])
+
+
+@pytest.mark.parametrize("K", [1, 2, 5, 50, 64, 65, 100, 128, 129, 200, 256])
+def test_neighbour_counts(oracle, K):
+    rng = np.random.default_rng(60 + K)
+    coords = rng.random((2500, 3)).astype(np.float32)
+    _check(oracle, K, coords, [0, 1200, 2500])
+
+
+@pytest.mark.parametrize("mbd", [2, 3, 4, 5])
+def test_max_bin_dims(oracle, mbd):
+    rng = np.random.default_rng(80 + mbd)
+    coords = rng.random((4000, 6)).astype(np.float32)
+    _check(oracle, 12, coords, [0, 4000], max_bin_dims=mbd)
+
+
+def test_reference_style_large(oracle):
+    # shape of the reference's own test (tests/test_binned_select_knn.py:95-163): N=10 000, K=50, three events
+    g = torch.Generator().manual_seed(45)
+    for D in (3, 8):
+        coords = torch.rand((10000, D), generator=g).numpy()
+        rs = [0, 3333, 5000, 10000]
+        gi, gd = _check(oracle, 50, coords, rs)
+        # and against cdist + topk exactly as the reference's baseline does
+        c = torch.from_numpy(coords)
+        for a, b in zip(rs[:-1], rs[1:]):
+            dm = torch.cdist(c[a:b], c[a:b], compute_mode="donot_use_mm_for_euclid_dist")
+            d, _ = torch.topk(dm, 50, largest=False)
+            ref = np.sort((d ** 2).numpy(), axis=1)
+            np.testing.assert_allclose(np.sort(gd[a:b], axis=1), ref, atol=1e-6, rtol=1e-4)
+
+
+def test_user_n_bins(oracle):
+    rng = np.random.default_rng(11)
+    coords = (rng.random((1000, 2)) - 0.5).astype(np.float32)
+    _check(oracle, 5, coords, [0, 1000], n_bins=torch.tensor(10, dtype=torch.int64, device="cuda"))
+    coords = (rng.random((1000, 4)) - 0.5).astype(np.float32)
+    _check(oracle, 10, coords, [0, 1000], n_bins=torch.tensor(10, dtype=torch.int64, device="cuda"))
+    _check(oracle, 8, rng.standard_normal((100, 3)).astype(np.float32), [0, 50, 100],
+           n_bins=torch.tensor(4, dtype=torch.int64, device="cuda"))
+
+
+def test_small_and_empty_events(oracle):
+    rng = np.random.default_rng(12)
+    coords = rng.random((300, 3)).astype(np.float32)
+    rs = [0, 3, 3, 40, 41, 300]   # events of 3, 0, 37, 1, 259 points with K = 20
+    gi, gd = _check(oracle, 20, coords, rs)
+    check_knn_properties(gi, gd, coords, rs, 20)
+    assert (gi[:3, 3:] == -1).all() and (gd[:3, 3:] == 0).all()
+    ti, td = _gpu_knn(20, coords, rs, torch_compatible_indices=True)
+    oi, od = oracle.binned_select_knn(20, coords, rs, torch_compatible_indices=True)
+    assert_knn_equal(ti, td, oi, od)
+    assert (ti[:3, 3:] == np.arange(3)[:, None]).all()
+
+
+def test_direction(oracle):
+    rng = np.random.default_rng(13)
+    coords = rng.random((4000, 3)).astype(np.float32)
+    direction = rng.integers(0, 4, size=4000).astype(np.int64)   # 3 = unconstrained
+    _check(oracle, 16, coords, [0, 1500, 4000], direction=direction)
+
+
+def test_duplicates_and_ties(oracle):
+    rng = np.random.default_rng(14)
+    base = rng.random((200, 3)).astype(np.float32)
+    coords = np.concatenate([base, base, base[:50], np.round(rng.random((500, 3)) * 8) / 8]).astype(np.float32)
+    gi, gd = _gpu_knn(10, coords, [0, coords.shape[0]])
+    oi, od = oracle.binned_select_knn(10, coords, [0, coords.shape[0]])
+    np.testing.assert_array_equal(np.sort(gd, axis=1), np.sort(od, axis=1))
+    check_knn_properties(gi, gd, coords, [0, coords.shape[0]], 10)
+
+
+def test_int32_row_splits_and_double_coords(oracle):
+    from fastgraphcompute_amd import binned_select_knn
+    rng = np.random.default_rng(15)
+    coords = rng.random((2000, 3))
+    rs = torch.tensor([0, 900, 2000], dtype=torch.int32, device="cuda")
+    idx, dist = binned_select_knn(7, torch.as_tensor(coords, device="cuda"), rs)
+    oi, od = oracle.binned_select_knn(7, coords.astype(np.float32), [0, 900, 2000])
+    assert_knn_equal(idx.cpu().numpy(), dist.cpu().numpy(), oi, od)
+
+
+def test_argument_errors():
+    from fastgraphcompute_amd import binned_select_knn
+    rs = torch.tensor([0, 10], device="cuda")
+    with pytest.raises(ValueError):
+        binned_select_knn(3, torch.rand(10, 0, device="cuda"), rs)
+    with pytest.raises(ValueError):
+        binned_select_knn(3, torch.rand(10, 3, device="cuda"), rs, max_bin_dims=0)
+    with pytest.raises(ValueError):   # one coordinate: unsupported number of binning dimensions
+        binned_select_knn(3, torch.rand(10, 1, device="cuda"), rs)
+    with pytest.raises(RuntimeError):  # row splits do not cover the points
+        binned_select_knn(3, torch.rand(10, 3, device="cuda"), torch.tensor([0, 8], device="cuda"))
+    c = torch.rand(10, 3, device="cuda")
+    c[0, 0] = float("inf")
+    with pytest.raises(RuntimeError):
+        binned_select_knn(3, c, rs)
+    with pytest.raises(RuntimeError):
+        binned_select_knn(3, torch.rand(10, 3), torch.tensor([0, 10]))
