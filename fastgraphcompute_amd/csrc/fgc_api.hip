@@ -19,7 +19,7 @@ extern "C" const char *fgc_error_string(int code)
 
 namespace {
 struct KnnWorkspace {
-    size_t geom, partial, keys, vals, sort, bb, sc, sdir, total;
+    size_t geom, partial, keys, vals, sort, sort_alt_vals, bb, sc, sdir, total;
     int ldc;
 };
 
@@ -47,6 +47,7 @@ KnnWorkspace plan(int64_t n, int D, int nbd, const int64_t *n_bins, int n_rs, bo
     w.keys = take((size_t)n * 4);
     w.vals = take((size_t)n * 4);
     w.sort = take(fgc_sort_workspace_bytes(n));
+    w.sort_alt_vals = fgc_align((size_t)n * 4);  // offset of the alternate value buffer inside the sort area
     w.bb = take((size_t)(B + 1) * 4);
     w.sc = take((size_t)w.ldc * D * 4);
     w.sdir = take(with_dir ? (size_t)n : 0);
@@ -63,12 +64,17 @@ extern "C" size_t fgc_binned_select_knn_workspace_bytes(int64_t n_vert, int32_t 
     return plan(n_vert, n_coords, n_bin_dims, n_bins, n_rs, true).total;
 }
 
-extern "C" int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
-                                         const int64_t *d_row_splits, const int64_t *row_splits_host,
-                                         int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
-                                         const int64_t *d_direction, int32_t tf_compat, int64_t *d_idx,
-                                         float *d_distsq, int32_t *d_status, uint64_t *d_stats, void *d_ws,
-                                         size_t ws_bytes, void *stream)
+namespace {
+struct KnnCall {
+    KnnWorkspace w;
+    int64_t B;
+    int key_bits;
+};
+
+// argument validation shared by the staged and the whole-call entry points
+int knn_validate(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host, int32_t n_rs, int32_t K,
+                 int32_t n_bin_dims, const int64_t *n_bins, bool with_dir, const void *d_ws, size_t ws_bytes,
+                 KnnCall *c)
 {
     if (n_vert < 0 || n_coords < 1 || n_rs < 2 || !row_splits_host || !n_bins) return FGC_EINVAL;
     if (K < 1 || K > FGC_MAX_K) return FGC_EINVAL;
@@ -78,13 +84,39 @@ extern "C" int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, 
     if (row_splits_host[0] != 0 || row_splits_host[n_rs - 1] != n_vert) return FGC_EINVAL;
     for (int r = 1; r < n_rs; r++)
         if (row_splits_host[r] < row_splits_host[r - 1]) return FGC_EINVAL;
-    if (n_vert == 0) return FGC_OK;
-    if (!d_coords || !d_row_splits || !d_idx || !d_distsq || !d_ws) return FGC_EINVAL;
-    const int64_t B = total_bins(n_bin_dims, n_bins, n_rs);
-    if (B < 0 || B >= (1ll << 31)) return FGC_EINVAL;
-    const KnnWorkspace w = plan(n_vert, n_coords, n_bin_dims, n_bins, n_rs, d_direction != nullptr);
-    if (ws_bytes < w.total) return FGC_ENOSPACE;
+    c->B = total_bins(n_bin_dims, n_bins, n_rs);
+    if (c->B < 0 || c->B >= (1ll << 31)) return FGC_EINVAL;
+    c->w = plan(n_vert > 0 ? n_vert : 1, n_coords, n_bin_dims, n_bins, n_rs, with_dir);
+    c->key_bits = 1;
+    while ((1ll << c->key_bits) < c->B) c->key_bits++;
+    if (n_vert > 0 && (!d_ws || ws_bytes < c->w.total)) return d_ws ? FGC_ENOSPACE : FGC_EINVAL;
+    return FGC_OK;
+}
 
+// where the sorted keys / order end up after the ping-pong passes of the sort
+void sorted_buffers(const KnnCall &c, char *ws, uint32_t **skeys, uint32_t **order)
+{
+    const int passes = (c.key_bits + 7) / 8;
+    const bool in_alt = (passes & 1) != 0;
+    char *sortws = ws + c.w.sort;
+    *skeys = in_alt ? (uint32_t *)sortws : (uint32_t *)(ws + c.w.keys);
+    *order = in_alt ? (uint32_t *)(sortws + c.w.sort_alt_vals) : (uint32_t *)(ws + c.w.vals);
+}
+}  // namespace
+
+extern "C" int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
+                                          const int64_t *d_row_splits, const int64_t *row_splits_host,
+                                          int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
+                                          const int64_t *d_direction, int32_t *d_status, void *d_ws,
+                                          size_t ws_bytes, void *stream)
+{
+    KnnCall c;
+    int rc = knn_validate(n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins, d_direction != nullptr,
+                          d_ws, ws_bytes, &c);
+    if (rc) return rc;
+    if (n_vert == 0) return FGC_OK;
+    if (!d_coords || !d_row_splits) return FGC_EINVAL;
+    const KnnWorkspace &w = c.w;
     hipStream_t s = (hipStream_t)stream;
     char *ws = (char *)d_ws;
     float *geom = (float *)(ws + w.geom);
@@ -93,25 +125,58 @@ extern "C" int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, 
     float *sc = (float *)(ws + w.sc);
     unsigned char *sdir = d_direction ? (unsigned char *)(ws + w.sdir) : nullptr;
 
-    int rc = fgc_bin_geometry_f32(d_coords, n_vert, n_coords, n_bin_dims, 0, n_bins, 1, 0.f, 0, geom, d_status,
-                                  ws + w.partial, fgc_bin_geometry_workspace_bytes(n_vert), stream);
+    rc = fgc_bin_geometry_f32(d_coords, n_vert, n_coords, n_bin_dims, 0, n_bins, 1, 0.f, 0, geom, d_status,
+                              ws + w.partial, fgc_bin_geometry_workspace_bytes(n_vert), stream);
     if (rc) return rc;
     rc = fgc_launch_bin_keys(d_coords, (int)n_vert, n_coords, n_bin_dims, geom, d_row_splits, n_rs, keys,
                              d_status, s);
     if (rc) return rc;
-    int key_bits = 1;
-    while ((1ll << key_bits) < B) key_bits++;
     uint32_t *skeys = nullptr, *order = nullptr;
-    rc = fgc_sort_keys(keys, vals, n_vert, key_bits, ws + w.sort, s, &skeys, &order);
+    rc = fgc_sort_keys(keys, vals, n_vert, c.key_bits, ws + w.sort, s, &skeys, &order);
     if (rc) return rc;
-    rc = fgc_launch_bin_boundaries(skeys, (int)n_vert, (int)B, bb, s);
+    uint32_t *skeys2, *order2;
+    sorted_buffers(c, ws, &skeys2, &order2);
+    if (skeys2 != skeys || order2 != order) return FGC_EINVAL;  // internal layout mismatch
+    rc = fgc_launch_bin_boundaries(skeys, (int)n_vert, (int)c.B, bb, s);
     if (rc) return rc;
-    rc = fgc_launch_gather_sorted(d_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir, s);
-    if (rc) return rc;
+    return fgc_launch_gather_sorted(d_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir, s);
+}
 
+extern "C" int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
+                                         int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
+                                         int32_t with_direction, int32_t tf_compat, int64_t *d_idx,
+                                         float *d_distsq, uint64_t *d_stats, void *d_ws, size_t ws_bytes,
+                                         void *stream)
+{
+    KnnCall c;
+    int rc = knn_validate(n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins, with_direction != 0,
+                          d_ws, ws_bytes, &c);
+    if (rc) return rc;
+    if (n_vert == 0) return FGC_OK;
+    if (!d_idx || !d_distsq) return FGC_EINVAL;
+    char *ws = (char *)d_ws;
     KnnArgs a;
-    a.sc = sc; a.ldc = w.ldc; a.skeys = skeys; a.order = order; a.bb = bb; a.geom = geom; a.sdir = sdir;
+    uint32_t *skeys, *order;
+    sorted_buffers(c, ws, &skeys, &order);
+    a.sc = (const float *)(ws + c.w.sc); a.ldc = c.w.ldc; a.skeys = skeys; a.order = order;
+    a.bb = (const int *)(ws + c.w.bb); a.geom = (const float *)(ws + c.w.geom);
+    a.sdir = with_direction ? (const unsigned char *)(ws + c.w.sdir) : nullptr;
     a.n = (int)n_vert; a.D = n_coords; a.nbd = n_bin_dims; a.K = K; a.tf_compat = tf_compat;
     a.out_idx = d_idx; a.out_dist = d_distsq; a.stats = (unsigned long long *)d_stats;
-    return fgc_launch_knn(a, s);
+    return fgc_launch_knn(a, (hipStream_t)stream);
+}
+
+extern "C" int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
+                                         const int64_t *d_row_splits, const int64_t *row_splits_host,
+                                         int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
+                                         const int64_t *d_direction, int32_t tf_compat, int64_t *d_idx,
+                                         float *d_distsq, int32_t *d_status, uint64_t *d_stats, void *d_ws,
+                                         size_t ws_bytes, void *stream)
+{
+    int rc = fgc_binned_knn_prepare_f32(d_coords, n_vert, n_coords, d_row_splits, row_splits_host, n_rs, K,
+                                        n_bin_dims, n_bins, d_direction, d_status, d_ws, ws_bytes, stream);
+    if (rc) return rc;
+    return fgc_binned_knn_search_f32(n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins,
+                                     d_direction != nullptr, tf_compat, d_idx, d_distsq, d_stats, d_ws, ws_bytes,
+                                     stream);
 }

@@ -122,6 +122,23 @@ int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_c
                               int64_t *d_idx, float *d_distsq, int32_t *d_status,
                               uint64_t *d_stats, void *d_ws, size_t ws_bytes, void *stream);
 
+/* The same forward in two stages sharing one workspace, for callers that
+ * search one prepared point set more than once or time the stages apart:
+ * prepare = geometry + binning + sort + bin boundaries + sorted coordinate
+ * copy (binned_knn_autograd_kernel.cpp:100-139); search = the neighbour
+ * search with the un-sort fused (:157-195).  Both take the same shape
+ * arguments; the workspace must not be touched in between. */
+int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
+                               const int64_t *d_row_splits, const int64_t *row_splits_host,
+                               int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
+                               const int64_t *d_direction, int32_t *d_status, void *d_ws,
+                               size_t ws_bytes, void *stream);
+int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
+                              int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
+                              int32_t with_direction, int32_t tf_compat, int64_t *d_idx,
+                              float *d_distsq, uint64_t *d_stats, void *d_ws, size_t ws_bytes,
+                              void *stream);
+
 /* ---------------------------------------------------------------------------
  * Replaces index_replacer_cuda_fn (index_replacer_cuda_kernel.cu:30-59):
  * out[i] = in[i] if in[i] < 0 or in[i] >= n_repl, else repl[in[i]].

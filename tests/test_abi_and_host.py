@@ -1,0 +1,97 @@
+"""CPU tests of the C-ABI library (loads, exports every declared symbol,
+rejects bad arguments before touching a device) and of the host-side logic."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "fgc_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fgc_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from fastgraphcompute_amd import _lib
+    L = _lib.lib()
+    names = _declared_symbols()
+    assert len(names) >= 12
+    for nm in names:
+        assert hasattr(L, nm), nm
+    assert set(names) == set(_lib.SIGNATURES.keys())
+    assert L.fgc_version() >= 100
+    assert b"binning dimensions" in L.fgc_error_string(-3)
+
+
+def test_argument_validation_without_device():
+    from fastgraphcompute_amd import _lib
+    L = _lib.lib()
+    fake = ctypes.c_void_p(4096)
+    nb = _lib.host_i64([10, 10, 10])
+    rs = _lib.host_i64([0, 100])
+    ws = L.fgc_binned_select_knn_workspace_bytes(100, 3, 3, nb, 2, 8)
+    assert ws > 0
+
+    def call(n=100, D=3, K=8, nbd=3, rs_=rs, n_rs=2, ws_bytes=ws, nb_=nb):
+        return L.fgc_binned_knn_search_f32(n, D, rs_, n_rs, K, nbd, nb_, 0, 0, fake, fake, None, fake, ws_bytes, None)
+    assert call(K=0) == -1 and call(K=257) == -1
+    assert call(nbd=1) == -3 and call(nbd=6) == -3 and call(D=2, nbd=3) == -3
+    assert call(rs_=_lib.host_i64([0, 99])) == -1            # row splits do not end at n_vert
+    assert call(rs_=_lib.host_i64([0, 120, 100]), n_rs=3) == -1
+    assert call(ws_bytes=16) == -2
+    assert call(nb_=_lib.host_i64([0, 10, 10])) == -1
+    assert call(n=0, rs_=_lib.host_i64([0, 0])) == 0          # empty input is a no-op
+    assert L.fgc_index_replacer_i64(fake, fake, fake, -1, 4, None) == -1
+    assert L.fgc_binned_select_knn_grad_f32(fake, fake, fake, fake, 10, 0, 3, None, None) == -1
+    assert L.fgc_gravnet_aggregate_fwd_f32(fake, fake, fake, fake, fake, None, 10, 4, 0, None) == -1
+
+
+def test_host_wrappers_reject_cpu_tensors_and_bad_arguments():
+    import fastgraphcompute_amd as fgc
+    with pytest.raises(RuntimeError):
+        fgc.binned_select_knn(3, torch.rand(10, 3), torch.tensor([0, 10]))
+    with pytest.raises(ValueError):
+        fgc.binned_select_knn(3, torch.rand(10, 0), torch.tensor([0, 10]))
+    with pytest.raises(ValueError):
+        fgc.binned_select_knn(3, torch.rand(10, 3), torch.tensor([0, 10]), max_bin_dims=0)
+    with pytest.raises(RuntimeError):
+        fgc.bin_by_coordinates(torch.rand(10, 3), torch.tensor([0, 10]), n_bins=4)
+    with pytest.raises(AssertionError):
+        fgc.index_replacer(torch.zeros(3, dtype=torch.int32), torch.zeros(3, dtype=torch.int64))
+    with pytest.raises(NotImplementedError):
+        fgc.oc_helper_matrices()
+
+
+def test_n_bins_heuristic_host():
+    from fastgraphcompute_amd.extensions.binned_select_knn import calculate_optimal_bins
+    from fastgraphcompute_amd.workloads import cfg5_many_events_d8
+    t = lambda v: torch.tensor(v, dtype=torch.int64)
+    assert calculate_optimal_bins(t([0, 6000, 10000]), 16, 3) == 18
+    assert calculate_optimal_bins(t([0, 50000, 100000, 150000, 200000]), 40, 3) == 30
+    assert calculate_optimal_bins(t([0, 1000000]), 64, 3) == 30
+    assert calculate_optimal_bins(torch.from_numpy(cfg5_many_events_d8()["row_splits"]).long(), 100, 3) == 13
+    assert calculate_optimal_bins(t([0, 3333, 5000, 10000]), 50, 3) == 11
+    assert calculate_optimal_bins(t([0, 50, 100]), 8, 3) == 5
+
+
+def test_workloads_are_deterministic():
+    from fastgraphcompute_amd import workloads
+    a, b = workloads.cfg4_zipf_blobs(0.01), workloads.cfg4_zipf_blobs(0.01)
+    assert a["coords"].dtype.name == "float32" and (a["coords"] == b["coords"]).all()
+    w5 = workloads.cfg5_many_events_d8()
+    assert w5["row_splits"][-1] == 500000 and len(w5["row_splits"]) == 65 and w5["coords"].shape == (500000, 8)
+    assert workloads.cfg2_blobs_4events(0.1)["coords"].shape == (20000, 4)
+
+
+def test_gravnet_module_state_dict_names():
+    from fastgraphcompute_amd.gnn_ops import GravNetOp
+    op = GravNetOp(8, 6, 3, 5, 4)
+    assert set(op.state_dict().keys()) == {
+        "space_transformations.weight", "space_transformations.bias", "propagate_transformations.weight",
+        "propagate_transformations.bias", "output_transformations.0.weight", "output_transformations.0.bias"}
+    assert op.output_transformations[0].in_features == 8 + 2 * 5
