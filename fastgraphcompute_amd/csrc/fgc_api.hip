@@ -1,6 +1,7 @@
 // Whole-call entry points and bookkeeping of libfgc_hip.so.
 #include "fgc_common.h"
 #include "fgc_internal.h"
+#include <cstdlib>
 
 extern "C" int fgc_version(void) { return 100; }
 
@@ -19,7 +20,7 @@ extern "C" const char *fgc_error_string(int code)
 
 namespace {
 struct KnnWorkspace {
-    size_t geom, partial, keys, vals, sort, sort_alt_vals, bb, sc, sdir, total;
+    size_t geom, partial, keys, vals, sort, sort_alt_vals, bb, sc, sdir, box_lo, box_hi, total;
     int ldc;
 };
 
@@ -51,6 +52,8 @@ KnnWorkspace plan(int64_t n, int D, int nbd, const int64_t *n_bins, int n_rs, bo
     w.bb = take((size_t)(B + 1) * 4);
     w.sc = take((size_t)w.ldc * D * 4);
     w.sdir = take(with_dir ? (size_t)n : 0);
+    w.box_lo = take((size_t)(w.ldc / 64) * D * 4);
+    w.box_hi = take((size_t)(w.ldc / 64) * D * 4);
     w.total = off;
     return w;
 }
@@ -68,8 +71,20 @@ namespace {
 struct KnnCall {
     KnnWorkspace w;
     int64_t B;
-    int key_bits;
+    int sub_bits;   // Morton bits per binned dimension appended to the flat bin in the sort key
+    int key_bits;   // total significant bits of the sort key
 };
+
+// bits per binned dimension for the in-bin Morton order: as many as fit into a 32-bit key, at most 5
+int choose_sub_bits(int bin_bits, int nbd)
+{
+    int sb = (32 - bin_bits) / nbd;
+    if (sb > 5) sb = 5;
+    if (sb < 0) sb = 0;
+    const char *e = getenv("FGC_SUB_BITS");   // tuning override
+    if (e && *e) { int v = atoi(e); if (v >= 0 && v * nbd + bin_bits <= 32) sb = v; }
+    return sb;
+}
 
 // argument validation shared by the staged and the whole-call entry points
 int knn_validate(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host, int32_t n_rs, int32_t K,
@@ -87,8 +102,10 @@ int knn_validate(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_hos
     c->B = total_bins(n_bin_dims, n_bins, n_rs);
     if (c->B < 0 || c->B >= (1ll << 31)) return FGC_EINVAL;
     c->w = plan(n_vert > 0 ? n_vert : 1, n_coords, n_bin_dims, n_bins, n_rs, with_dir);
-    c->key_bits = 1;
-    while ((1ll << c->key_bits) < c->B) c->key_bits++;
+    int bin_bits = 1;
+    while ((1ll << bin_bits) < c->B) bin_bits++;
+    c->sub_bits = choose_sub_bits(bin_bits, n_bin_dims);
+    c->key_bits = bin_bits + c->sub_bits * n_bin_dims;
     if (n_vert > 0 && (!d_ws || ws_bytes < c->w.total)) return d_ws ? FGC_ENOSPACE : FGC_EINVAL;
     return FGC_OK;
 }
@@ -128,8 +145,8 @@ extern "C" int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert,
     rc = fgc_bin_geometry_f32(d_coords, n_vert, n_coords, n_bin_dims, 0, n_bins, 1, 0.f, 0, geom, d_status,
                               ws + w.partial, fgc_bin_geometry_workspace_bytes(n_vert), stream);
     if (rc) return rc;
-    rc = fgc_launch_bin_keys(d_coords, (int)n_vert, n_coords, n_bin_dims, geom, d_row_splits, n_rs, keys,
-                             d_status, s);
+    rc = fgc_launch_bin_keys(d_coords, (int)n_vert, n_coords, n_bin_dims, c.sub_bits, geom, d_row_splits, n_rs,
+                             keys, d_status, s);
     if (rc) return rc;
     uint32_t *skeys = nullptr, *order = nullptr;
     rc = fgc_sort_keys(keys, vals, n_vert, c.key_bits, ws + w.sort, s, &skeys, &order);
@@ -137,9 +154,12 @@ extern "C" int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert,
     uint32_t *skeys2, *order2;
     sorted_buffers(c, ws, &skeys2, &order2);
     if (skeys2 != skeys || order2 != order) return FGC_EINVAL;  // internal layout mismatch
-    rc = fgc_launch_bin_boundaries(skeys, (int)n_vert, (int)c.B, bb, s);
+    rc = fgc_launch_bin_boundaries(skeys, (int)n_vert, c.sub_bits * n_bin_dims, (int)c.B, bb, s);
     if (rc) return rc;
-    return fgc_launch_gather_sorted(d_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir, s);
+    rc = fgc_launch_gather_sorted(d_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir, s);
+    if (rc) return rc;
+    return fgc_launch_chunk_boxes(sc, (int)n_vert, n_coords, w.ldc, (float *)(ws + w.box_lo),
+                                  (float *)(ws + w.box_hi), s);
 }
 
 extern "C" int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
@@ -159,6 +179,9 @@ extern "C" int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const
     uint32_t *skeys, *order;
     sorted_buffers(c, ws, &skeys, &order);
     a.sc = (const float *)(ws + c.w.sc); a.ldc = c.w.ldc; a.skeys = skeys; a.order = order;
+    a.key_shift = c.sub_bits * n_bin_dims;
+    a.box_lo = (const float *)(ws + c.w.box_lo); a.box_hi = (const float *)(ws + c.w.box_hi);
+    a.n_chunks = c.w.ldc / 64;
     a.bb = (const int *)(ws + c.w.bb); a.geom = (const float *)(ws + c.w.geom);
     a.sdir = with_direction ? (const unsigned char *)(ws + c.w.sdir) : nullptr;
     a.n = (int)n_vert; a.D = n_coords; a.nbd = n_bin_dims; a.K = K; a.tf_compat = tf_compat;

@@ -280,10 +280,13 @@ extern "C" int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t
 }
 
 // ---------------------------------------------------------------------------
-// sort keys for the kNN pipeline: key = flat bin (uint32)
+// sort keys for the kNN pipeline: key = (flat bin << sub_bits*nbd) | Morton code
+// of the point's position inside its bin (sub_bits per binned dimension).  The
+// Morton part only orders points inside a bin so that consecutive points are
+// spatially compact; it never changes which bin a point belongs to.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void k_bin_keys(const float *__restrict__ coords, int n, int ld, int nbd,
-                                                  const float *__restrict__ geom,
+                                                  int sub_bits, const float *__restrict__ geom,
                                                   const int64_t *__restrict__ rs, int n_rs,
                                                   uint32_t *__restrict__ keys, int *__restrict__ status)
 {
@@ -292,16 +295,29 @@ __global__ __launch_bounds__(256) void k_bin_keys(const float *__restrict__ coor
     BinGeom g = load_geom(geom);
     int clamped = 0;
     uint32_t f = 0, stride = 1;
+    int sub[FGC_MAX_BIN_DIMS];
+    const int smax = (1 << sub_bits) - 1;
 #pragma unroll
-    for (int d = FGC_MAX_BIN_DIMS - 1; d >= 0; d--)
+    for (int d = FGC_MAX_BIN_DIMS - 1; d >= 0; d--) {
+        sub[d] = 0;
         if (d < nbd) {
-            int b = bin_of(coords[(int64_t)v * ld + d], g.mn[d], g.bw, g.nb[d], clamped);
+            const float x = coords[(int64_t)v * ld + d];
+            int b = bin_of(x, g.mn[d], g.bw, g.nb[d], clamped);
             f += (uint32_t)b * stride;
             stride *= (uint32_t)g.nb[d];
+            const float t = (x - g.mn[d]) / g.bw + 1e-3f;
+            const float fr = t - (float)b;  // position inside the bin, [0, 1) unless the point was clamped
+            sub[d] = min(max((int)(fr * (float)(smax + 1)), 0), smax);
         }
+    }
     f += (uint32_t)event_of(rs, n_rs, v) * stride;
     if (clamped && status) atomicOr(&status[0], FGC_ST_CLAMPED);
-    keys[v] = f;
+    uint32_t code = 0;
+    for (int l = sub_bits - 1; l >= 0; l--)
+#pragma unroll
+        for (int d = 0; d < FGC_MAX_BIN_DIMS; d++)
+            if (d < nbd) code = (code << 1) | (uint32_t)((sub[d] >> l) & 1);
+    keys[v] = (f << (sub_bits * nbd)) | code;
 }
 
 // ---------------------------------------------------------------------------
@@ -339,33 +355,43 @@ __global__ __launch_bounds__(256) void k_rs_hist(const uint32_t *__restrict__ ke
     block_hist[threadIdx.x * nblk + blockIdx.x] = s_h[threadIdx.x];
 }
 
-// in-place exclusive scan of `len` uint32 values by one 1024-thread block;
+// in-place exclusive scan of `len` uint32 values by one 1024-thread block,
+// in coalesced tiles of 8192 values (8 consecutive values per thread);
 // if total != NULL it receives the sum
 __global__ __launch_bounds__(1024) void k_scan_excl_u32(uint32_t *__restrict__ a, int len,
                                                         uint32_t *__restrict__ total)
 {
     __shared__ uint32_t s_w[16];
+    __shared__ uint32_t s_carry;
     const int t = threadIdx.x, lane = t & 63, wv = t >> 6;
-    const int per = (len + 1023) / 1024;
-    const int lo = min(len, t * per), hi = min(len, lo + per);
-    uint32_t sum = 0;
-    for (int i = lo; i < hi; i++) sum += a[i];
-    uint32_t incl = sum;
-    for (int o = 1; o < 64; o <<= 1) {
-        uint32_t u = __shfl_up(incl, o, 64);
-        if (lane >= o) incl += u;
-    }
-    if (lane == 63) s_w[wv] = incl;
+    if (t == 0) s_carry = 0;
     __syncthreads();
-    uint32_t woff = 0;
-    for (int w = 0; w < wv; w++) woff += s_w[w];
-    uint32_t run = woff + incl - sum;
-    for (int i = lo; i < hi; i++) {
-        uint32_t v = a[i];
-        a[i] = run;
-        run += v;
+    for (int base = 0; base < len; base += 8192) {
+        const int i0 = base + t * 8;
+        uint32_t v[8];
+        uint32_t sum = 0;
+#pragma unroll
+        for (int k = 0; k < 8; k++) { v[k] = (i0 + k < len) ? a[i0 + k] : 0u; sum += v[k]; }
+        uint32_t incl = sum;
+        for (int o = 1; o < 64; o <<= 1) {
+            uint32_t u = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += u;
+        }
+        if (lane == 63) s_w[wv] = incl;
+        __syncthreads();
+        uint32_t woff = s_carry;
+        for (int w = 0; w < wv; w++) woff += s_w[w];
+        uint32_t run = woff + incl - sum;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            if (i0 + k < len) a[i0 + k] = run;
+            run += v[k];
+        }
+        __syncthreads();
+        if (t == 1023) s_carry = run;
+        __syncthreads();
     }
-    if (total && t == 1023) *total = run;
+    if (total && t == 0) *total = s_carry;
 }
 
 __global__ __launch_bounds__(256) void k_rs_scatter(const uint32_t *__restrict__ keys_in,
@@ -460,13 +486,13 @@ int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void 
 }
 
 // bin_boundaries[b] = first sorted position whose key is >= b, for b in [0, n_bins_total]
-__global__ __launch_bounds__(256) void k_bin_boundaries(const uint32_t *__restrict__ skeys, int n,
+__global__ __launch_bounds__(256) void k_bin_boundaries(const uint32_t *__restrict__ skeys, int n, int shift,
                                                         int n_bins_total, int *__restrict__ bb)
 {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i > n) return;
-    long long prev = (i > 0) ? (long long)skeys[i - 1] : -1ll;
-    long long cur = (i < n) ? (long long)skeys[i] : (long long)n_bins_total;
+    long long prev = (i > 0) ? (long long)(skeys[i - 1] >> shift) : -1ll;
+    long long cur = (i < n) ? (long long)(skeys[i] >> shift) : (long long)n_bins_total;
     if (cur > n_bins_total) cur = n_bins_total;
     for (long long b = prev + 1; b <= cur; b++) bb[b] = i;
 }
@@ -488,19 +514,19 @@ __global__ __launch_bounds__(256) void k_gather_sorted(const float *__restrict__
     }
 }
 
-int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, const float *d_geom,
+int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, int sub_bits, const float *d_geom,
                         const int64_t *d_rs, int n_rs, uint32_t *d_keys, int *d_status, hipStream_t s)
 {
     hipLaunchKernelGGL(k_bin_keys, dim3((unsigned)fgc_cdiv(n, 256)), dim3(256), 0, s, d_coords, n, ld, nbd,
-                       d_geom, d_rs, n_rs, d_keys, d_status);
+                       sub_bits, d_geom, d_rs, n_rs, d_keys, d_status);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
 
-int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int n_bins_total, int *bb, hipStream_t s)
+int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int shift, int n_bins_total, int *bb, hipStream_t s)
 {
     hipLaunchKernelGGL(k_bin_boundaries, dim3((unsigned)fgc_cdiv((int64_t)n + 1, 256)), dim3(256), 0, s, skeys,
-                       n, n_bins_total, bb);
+                       n, shift, n_bins_total, bb);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
@@ -510,6 +536,33 @@ int fgc_launch_gather_sorted(const float *coords, const uint32_t *order, int n, 
 {
     hipLaunchKernelGGL(k_gather_sorted, dim3((unsigned)fgc_cdiv(n, 256)), dim3(256), 0, s, coords, order, n,
                        D, ldc, sc, direction, sdir);
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
+}
+
+// axis-aligned bounding box of every 64 consecutive sorted points, all D coordinates:
+// box_lo[d * n_chunks + c], box_hi[d * n_chunks + c]
+__global__ __launch_bounds__(256) void k_chunk_boxes(const float *__restrict__ sc, int n, int D, int ldc,
+                                                     int n_chunks, float *__restrict__ box_lo,
+                                                     float *__restrict__ box_hi)
+{
+    const int lane = fgc_lane();
+    const int c = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
+    if (c >= n_chunks) return;
+    const int j = c * 64 + lane;
+    for (int d = 0; d < D; d++) {
+        const float x = (j < n) ? sc[(size_t)d * ldc + j] : NAN;
+        const float lo = wave_min_f((j < n) ? x : INFINITY);
+        const float hi = wave_max_f((j < n) ? x : -INFINITY);
+        if (lane == 0) { box_lo[(size_t)d * n_chunks + c] = lo; box_hi[(size_t)d * n_chunks + c] = hi; }
+    }
+}
+
+int fgc_launch_chunk_boxes(const float *sc, int n, int D, int ldc, float *box_lo, float *box_hi, hipStream_t s)
+{
+    const int n_chunks = ldc / 64;
+    hipLaunchKernelGGL(k_chunk_boxes, dim3((unsigned)fgc_cdiv(n_chunks, 4)), dim3(256), 0, s, sc, n, D, ldc,
+                       n_chunks, box_lo, box_hi);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
