@@ -63,10 +63,14 @@ def main():
     grad_d = torch.from_numpy(gd_h).to(dev)
     config.sync_checks = True
 
+    coords_g = coords.clone().requires_grad_(True)
+
     def step():
-        idx, dist = fgc.binned_select_knn(K, coords, rs)
-        g = binned_select_knn_grad(grad_d, idx, coords)
-        return idx, dist, g
+        # the user-visible path: forward through the autograd op, backward with the upstream gradient
+        idx, dist = fgc.binned_select_knn(K, coords_g, rs)
+        coords_g.grad = None
+        dist.backward(grad_d)
+        return idx, dist, coords_g.grad
 
     for _ in range(args.warmup):
         step()
@@ -118,7 +122,10 @@ def main():
     reps = max(3, args.steps)
     t_prep = float(np.mean(timed(prepare, reps)))
     t_knn = float(np.mean(timed(lambda: search(False), reps)))
-    t_grad = float(np.mean(timed(lambda: binned_select_knn_grad(grad_d, idx, coords), reps)))
+    order = torch.empty(n, dtype=torch.int32, device=dev)
+    _lib.check(L.fgc_binned_knn_export_order_i32(n, D, rs_arr, n_rs, K, nbd, nb_arr, 0, _lib.ptr(ws), ws_bytes,
+                                                 _lib.ptr(order), st))
+    t_grad = float(np.mean(timed(lambda: binned_select_knn_grad(grad_d, idx, coords, order), reps)))
 
     # algorithmic bytes of one search launch: every distance evaluation reads one
     # D-float candidate, every query is read once, every (idx, distsq) slot written once

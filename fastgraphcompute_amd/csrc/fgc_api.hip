@@ -189,6 +189,22 @@ extern "C" int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const
     return fgc_launch_knn(a, (hipStream_t)stream);
 }
 
+extern "C" int fgc_binned_knn_export_order_i32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
+                                               int32_t n_rs, int32_t K, int32_t n_bin_dims,
+                                               const int64_t *n_bins, int32_t with_direction, const void *d_ws,
+                                               size_t ws_bytes, int32_t *d_order_out, void *stream)
+{
+    KnnCall c;
+    int rc = knn_validate(n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins, with_direction != 0,
+                          d_ws, ws_bytes, &c);
+    if (rc) return rc;
+    if (n_vert == 0) return FGC_OK;
+    if (!d_order_out) return FGC_EINVAL;
+    uint32_t *skeys, *order;
+    sorted_buffers(c, (char *)const_cast<void *>(d_ws), &skeys, &order);
+    return fgc_copy_u32(d_order_out, order, n_vert, (hipStream_t)stream);
+}
+
 extern "C" int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
                                          const int64_t *d_row_splits, const int64_t *row_splits_host,
                                          int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,

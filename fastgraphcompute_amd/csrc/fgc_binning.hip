@@ -24,6 +24,24 @@ int fgc_fill_u32(void *d, uint32_t v, int64_t n_words, hipStream_t s)
     return FGC_OK;
 }
 
+__global__ void k_copy_u32(uint32_t *__restrict__ dst, const uint32_t *__restrict__ src, int64_t n)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] = src[i];
+}
+
+int fgc_copy_u32(void *dst, const void *src, int64_t n_words, hipStream_t s)
+{
+    if (n_words <= 0) return FGC_OK;
+    int64_t blocks = fgc_cdiv(n_words, 256 * 8);
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(k_copy_u32, dim3((unsigned)blocks), dim3(256), 0, s, (uint32_t *)dst, (const uint32_t *)src,
+                       n_words);
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
+}
+
 __device__ __forceinline__ float wave_min_f(float v)
 {
     for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, 64));

@@ -49,3 +49,4 @@ __device__ __forceinline__ int fgc_mbcnt(unsigned long long m)
 
 // internal launchers shared between translation units (all enqueue on `s`)
 int fgc_fill_u32(void *d, uint32_t v, int64_t n_words, hipStream_t s);
+int fgc_copy_u32(void *dst, const void *src, int64_t n_words, hipStream_t s);

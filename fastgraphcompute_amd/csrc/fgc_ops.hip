@@ -30,67 +30,113 @@ extern "C" int fgc_index_replacer_i64(const int64_t *d_in, const int64_t *d_repl
 // ---------------------------------------------------------------------------
 // gradient of distsq wrt the coordinates
 // ---------------------------------------------------------------------------
-// A group of W = 2^w lanes (W >= min(K, 64)) owns one query; lane k of the
-// group owns neighbour slot k (K > 64: slots k, k + 64, ...).  The neighbour
-// receives +2 g (x_m - x_i) through a float atomic; the query's own
-// -2 sum_k g (x_m - x_i) is reduced inside the group first and added with one
-// atomic per coordinate.
-template <int W>
+// g[m] += 2 gd[i,k] (x_m - x_i) for every neighbour m = idx[i,k] and
+// g[i] -= sum_k of the same terms.  A block takes GQ queries - consecutive in
+// the bin-sorted order when `order` is given, so their neighbourhoods overlap -
+// and first combines all contributions to the same target point in an LDS hash
+// table (open addressing, LDS float atomics); only the distinct targets go to
+// global memory, one float atomic per coordinate.  Pairs that find no slot
+// within a few probes go to global memory directly.
+#define GQ 64          // queries per block (4 wavefronts x 16)
+#define GRAD_PROBES 8
+#define GRAD_EMPTY 0xffffffffu
+
 __global__ __launch_bounds__(256) void k_knn_grad(const float *__restrict__ gd, const int64_t *__restrict__ idx,
                                                   const float *__restrict__ x, float *__restrict__ gx,
-                                                  int64_t n, int K, int D, int *__restrict__ status)
+                                                  const uint32_t *__restrict__ order, int64_t n, int K, int D,
+                                                  int H, int *__restrict__ status)
 {
-    constexpr int QPW = 64 / W;  // queries per wave
-    const int lane = fgc_lane();
-    const int sub = lane / W, kl = lane % W;
-    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    const int64_t i = wave * QPW + sub;
-    const bool qv = i < n;
+    extern __shared__ unsigned char s_raw[];
+    unsigned *keys = (unsigned *)s_raw;            // [H]
+    float *vals = (float *)(s_raw + (size_t)H * 4);  // [H][D]
+    for (int t = threadIdx.x; t < H; t += 256) keys[t] = GRAD_EMPTY;
+    for (int t = threadIdx.x; t < H * D; t += 256) vals[t] = 0.f;
+    __syncthreads();
+
+    const int lane = fgc_lane(), wv = threadIdx.x >> 6;
+    const unsigned hmask = (unsigned)H - 1u;
     bool bad = false;
-    for (int c = 0; c < D; c++) {
-        const float xi = qv ? x[i * D + c] : 0.f;
-        float self = 0.f;
-        for (int k = kl; k < K; k += W) {
-            if (!qv) continue;
-            const int64_t m = idx[i * K + k];
-            if (m < 0) continue;
-            if (m >= n) { bad = true; continue; }
-            const float g = gd[i * K + k];
-            const float add = 2.f * g * (x[m * D + c] - xi);
-            self -= add;
-            atomicAdd(&gx[m * D + c], add);
+
+    // add v[0..D) to target m: LDS table if a slot is found, global memory otherwise
+    auto slot_of = [&](unsigned m) -> int {
+        unsigned h = (m * 2654435761u) >> 7;
+        for (int p = 0; p < GRAD_PROBES; p++) {
+            const unsigned sl = (h + p) & hmask;
+            const unsigned old = atomicCAS(&keys[sl], GRAD_EMPTY, m);
+            if (old == GRAD_EMPTY || old == m) return (int)sl;
         }
+        return -1;
+    };
+
+    for (int qq = wv; qq < GQ; qq += 4) {
+        const int64_t pos = (int64_t)blockIdx.x * GQ + qq;
+        if (pos >= n) break;   // wave-uniform
+        const int64_t i = order ? (int64_t)order[pos] : pos;
+        // the query's own slot (its contribution is the negated sum over its row)
+        int self_slot = 0;
+        if (lane == 0) self_slot = slot_of((unsigned)i);
+        self_slot = fgc_readlane_i(self_slot, 0);
+        for (int k0 = 0; k0 < K; k0 += 64) {
+            const int k = k0 + lane;
+            int64_t m = -1;
+            float g = 0.f;
+            if (k < K) { m = idx[i * K + k]; g = gd[i * K + k]; }
+            if (m >= n) { bad = true; m = -1; }
+            const bool on = m >= 0;
+            const int sl = on ? slot_of((unsigned)m) : -1;
+            for (int c = 0; c < D; c++) {
+                const float xi = x[i * D + c];
+                float add = 0.f;
+                if (on) {
+                    add = 2.f * g * (x[m * D + c] - xi);
+                    if (sl >= 0) atomicAdd(&vals[sl * D + c], add);
+                    else atomicAdd(&gx[m * D + c], add);
+                }
+                float self = add;
 #pragma unroll
-        for (int o = W / 2; o > 0; o >>= 1) self += __shfl_xor(self, o, 64);
-        if (qv && kl == 0) atomicAdd(&gx[i * D + c], self);
+                for (int o = 32; o > 0; o >>= 1) self += __shfl_xor(self, o, 64);
+                if (lane == 0) {
+                    if (self_slot >= 0) atomicAdd(&vals[self_slot * D + c], -self);
+                    else atomicAdd(&gx[i * D + c], -self);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t < H; t += 256) {
+        const unsigned m = keys[t];
+        if (m == GRAD_EMPTY) continue;
+        for (int c = 0; c < D; c++) {
+            const float v = vals[t * D + c];
+            if (v != 0.f) atomicAdd(&gx[(int64_t)m * D + c], v);
+        }
     }
     if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
 }
 
+static int grad_table_size(int D)
+{
+    int H = 2048;
+    while (H > 64 && (size_t)H * (4 + 4 * (size_t)D) > 40960) H >>= 1;
+    return H;
+}
+
 extern "C" int fgc_binned_select_knn_grad_f32(const float *d_grad_distsq, const int64_t *d_idx,
                                               const float *d_coords, float *d_grad_coords, int64_t n_vert,
-                                              int32_t K, int32_t n_coords, int32_t *d_status, void *stream)
+                                              int32_t K, int32_t n_coords, const int32_t *d_order,
+                                              int32_t *d_status, void *stream)
 {
-    if (n_vert < 0 || K < 1 || n_coords < 1) return FGC_EINVAL;
+    if (n_vert < 0 || K < 1 || n_coords < 1 || n_coords > 2048) return FGC_EINVAL;
+    if (n_vert >= (1ll << 32) - 1) return FGC_EINVAL;
     if (n_vert == 0) return FGC_OK;
     hipStream_t s = (hipStream_t)stream;
     int rc = fgc_fill_u32(d_grad_coords, 0u, n_vert * n_coords, s);
     if (rc) return rc;
-    int W = 64;
-    while (W > 8 && (W >> 1) >= K) W >>= 1;
-    const int qpw = 64 / W;
-    const int64_t waves = fgc_cdiv(n_vert, qpw);
-    const unsigned blocks = (unsigned)fgc_cdiv(waves, 4);
-#define FGC_GRAD_LAUNCH(WW)                                                                              \
-    hipLaunchKernelGGL((k_knn_grad<WW>), dim3(blocks), dim3(256), 0, s, d_grad_distsq, d_idx, d_coords, \
-                       d_grad_coords, n_vert, (int)K, (int)n_coords, d_status)
-    switch (W) {
-    case 8: FGC_GRAD_LAUNCH(8); break;
-    case 16: FGC_GRAD_LAUNCH(16); break;
-    case 32: FGC_GRAD_LAUNCH(32); break;
-    default: FGC_GRAD_LAUNCH(64); break;
-    }
-#undef FGC_GRAD_LAUNCH
+    const int H = grad_table_size(n_coords);
+    const size_t lds = (size_t)H * (4 + 4 * (size_t)n_coords);
+    const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GQ);
+    hipLaunchKernelGGL(k_knn_grad, dim3(blocks), dim3(256), lds, s, d_grad_distsq, d_idx, d_coords,
+                       d_grad_coords, (const uint32_t *)d_order, n_vert, (int)K, (int)n_coords, H, d_status);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }

@@ -63,6 +63,7 @@ class _BinnedKNN(torch.autograd.Function):
         rs_dev = rs_dev.contiguous()
         idx = torch.empty((n, K), dtype=torch.int64, device=dev)
         dist = torch.empty((n, K), dtype=torch.float32, device=dev)
+        order = None
         if n > 0:
             nb_arr = _lib.host_i64(nb)
             rs_arr = _lib.host_i64(rs_list)
@@ -78,6 +79,12 @@ class _BinnedKNN(torch.autograd.Function):
                     _lib.ptr(coords), n, D, _lib.ptr(rs_dev), rs_arr, n_rs, K, nbd, nb_arr, _lib.ptr(dirt),
                     1 if tf_compat else 0, _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(status), _lib.ptr(stats),
                     _lib.ptr(ws), ws_bytes, _lib.stream_ptr()))
+            if coords.requires_grad:
+                order = torch.empty(n, dtype=torch.int32, device=dev)
+                with torch.cuda.device(dev):
+                    _lib.check(L.fgc_binned_knn_export_order_i32(n, D, rs_arr, n_rs, K, nbd, nb_arr,
+                                                                 1 if dirt is not None else 0, _lib.ptr(ws), ws_bytes,
+                                                                 _lib.ptr(order), _lib.stream_ptr()))
             if config.sync_checks:
                 flags = int(status[0].item())
                 if flags & _lib.ST_NONFINITE:
@@ -88,23 +95,30 @@ class _BinnedKNN(torch.autograd.Function):
                 s = stats.tolist()
                 last_stats.update(distance_evaluations=s[0], candidate_chunks=s[1], insertions=s[2],
                                   n_bins=nb, n_vert=n, K=K, n_coords=D)
-        ctx.save_for_backward(idx, coords)
+        if order is None:
+            order = torch.empty(0, dtype=torch.int32, device=dev)
+        ctx.save_for_backward(idx, coords, order)
         ctx.mark_non_differentiable(idx)
         return idx, dist
 
     @staticmethod
     def backward(ctx, _grad_idx, grad_dist):
-        idx, coords = ctx.saved_tensors
+        idx, coords, order = ctx.saved_tensors
         if not ctx.needs_input_grad[0]:
             return None, None, None, None, None, None, None
         if grad_dist is None:
             return torch.zeros_like(coords), None, None, None, None, None, None
-        return binned_select_knn_grad(grad_dist, idx, coords), None, None, None, None, None, None
+        g = binned_select_knn_grad(grad_dist, idx, coords, order if order.numel() else None)
+        return g, None, None, None, None, None, None
 
 
-def binned_select_knn_grad(grad_distsq: torch.Tensor, idx: torch.Tensor, coords: torch.Tensor) -> torch.Tensor:
+def binned_select_knn_grad(grad_distsq: torch.Tensor, idx: torch.Tensor, coords: torch.Tensor,
+                           order: Optional[torch.Tensor] = None) -> torch.Tensor:
     """d loss / d coords from d loss / d distsq
-    (binned_select_knn_grad_cuda_fn, binned_select_knn_grad_cuda_kernel.cu:90-164)."""
+    (binned_select_knn_grad_cuda_fn, binned_select_knn_grad_cuda_kernel.cu:90-164).
+    `order` (int32 [N], optional) is a spatially coherent processing order of the
+    points, e.g. the forward's bin-sorted order; it speeds the kernel up and does
+    not change the result beyond float summation order."""
     _lib.require_device(grad_distsq, idx, coords)
     L = _lib.lib()
     g = grad_distsq.to(torch.float32).contiguous()
@@ -115,8 +129,12 @@ def binned_select_knn_grad(grad_distsq: torch.Tensor, idx: torch.Tensor, coords:
     out = torch.empty((n, D), dtype=torch.float32, device=x.device)
     status = torch.zeros(4, dtype=torch.int32, device=x.device)
     with torch.cuda.device(x.device):
+        if order is not None:
+            order = order.to(device=x.device, dtype=torch.int32).contiguous()
+            if order.numel() != n:
+                raise ValueError("order must hold one entry per point")
         _lib.check(L.fgc_binned_select_knn_grad_f32(_lib.ptr(g), _lib.ptr(ii), _lib.ptr(x), _lib.ptr(out), n, K, D,
-                                                    _lib.ptr(status), _lib.stream_ptr()))
+                                                    _lib.ptr(order), _lib.ptr(status), _lib.stream_ptr()))
     return out
 
 

@@ -153,11 +153,25 @@ int fgc_index_replacer_i64(const int64_t *d_in, const int64_t *d_repl, int64_t *
  *   g[i,c]      = -2 sum_k gd[i,k] (x[n_ik,c] - x[i,c])
  *   g[n_ik,c]  +=  2 gd[i,k] (x[n_ik,c] - x[i,c])          (n_ik < 0 skipped)
  * d_grad_coords [n_vert, n_coords] is fully overwritten.
+ * d_order (optional, int32 [n_vert]): a permutation of the points in which
+ * consecutive entries are spatial neighbours (the bin-sorted order of the
+ * forward, see fgc_binned_knn_export_order_i32).  It only changes the order in
+ * which queries are processed, so that contributions to the same point are
+ * combined on chip before they reach memory; NULL = original order.
  */
 int fgc_binned_select_knn_grad_f32(const float *d_grad_distsq, const int64_t *d_idx,
                                    const float *d_coords, float *d_grad_coords,
                                    int64_t n_vert, int32_t K, int32_t n_coords,
-                                   int32_t *d_status, void *stream);
+                                   const int32_t *d_order, int32_t *d_status, void *stream);
+
+/* Copies the bin-sorted order (sorted position -> original row) out of a
+ * workspace that fgc_binned_knn_prepare_f32 / fgc_binned_select_knn_f32 filled
+ * with the same shape arguments.  No counterpart in the reference (its sort
+ * order, binned_knn_autograd_kernel.cpp:118-120, never leaves the forward). */
+int fgc_binned_knn_export_order_i32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
+                                    int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
+                                    int32_t with_direction, const void *d_ws, size_t ws_bytes,
+                                    int32_t *d_order_out, void *stream);
 
 /* ---------------------------------------------------------------------------
  * Replaces select_with_default (oc_helper.py:232-271) for float32 features:

@@ -47,7 +47,7 @@ def test_argument_validation_without_device():
     assert call(nb_=_lib.host_i64([0, 10, 10])) == -1
     assert call(n=0, rs_=_lib.host_i64([0, 0])) == 0          # empty input is a no-op
     assert L.fgc_index_replacer_i64(fake, fake, fake, -1, 4, None) == -1
-    assert L.fgc_binned_select_knn_grad_f32(fake, fake, fake, fake, 10, 0, 3, None, None) == -1
+    assert L.fgc_binned_select_knn_grad_f32(fake, fake, fake, fake, 10, 0, 3, None, None, None) == -1
     assert L.fgc_gravnet_aggregate_fwd_f32(fake, fake, fake, fake, fake, None, 10, 4, 0, None) == -1
 
 

@@ -75,6 +75,11 @@ def test_grad_vs_checker(oracle, n, D, K):
                                  torch.from_numpy(coords).cuda()).cpu().numpy()
     exp = oracle.knn_grad(gd, idx, coords)
     assert _rel_err(got, exp) < DIST_RTOL
+    # with a processing order (here: sorted by the first coordinate) the result is the same
+    order = torch.from_numpy(np.argsort(coords[:, 0], kind="stable").astype(np.int32)).cuda()
+    got_o = binned_select_knn_grad(torch.from_numpy(gd).cuda(), torch.from_numpy(idx).cuda(),
+                                   torch.from_numpy(coords).cuda(), order).cpu().numpy()
+    assert _rel_err(got_o, exp) < DIST_RTOL
     # float64 closed form: g_i = -2 sum_k gd_ik (x_n - x_i), g_n += 2 gd_ik (x_n - x_i)
     x = coords.astype(np.float64)
     ref = np.zeros_like(x)
