@@ -32,18 +32,28 @@
 // the same float operations as the distance itself, so it can never reject a
 // candidate the distance test would accept: the result is the exact kNN set of
 // the reference's shell search (binned_select_knn_cuda_kernel.cu:101-248).
+//
+// The whole search of a group is one loop over "spans" (seed spans first, then
+// one span per bin row) with a single copy of the chunk / pool code inside: the
+// kernel stays small in registers and instructions, which is what bounds its
+// occupancy.
 #include "fgc_common.h"
 #include "fgc_internal.h"
 
 #ifndef QT
 #define QT 8           // queries per wavefront
 #endif
-#define CULL_MIN 3     // ranges of at least this many chunks get the per-chunk box test
+#ifndef PRUNE_AT
+#define PRUNE_AT 32    // a pool is pruned when it holds this many candidates more than K
+#endif
+#define CULL_MIN 3     // spans of at least this many chunks get the per-chunk box test
 
 // wavefronts per block, chosen so that a block's pools fit the 64 KB static LDS limit
 template <int NSEG> struct KnnCfg { static constexpr int WPB = (NSEG <= 2 ? 2 : 1) * (16 / QT); };
 
-template <int DT, int NSEG>
+// DT: coordinates per point held in registers (0 = any number, read from memory)
+// NSEG: ceil(K / 64);  RD: bin-row dimensions (binned dimensions - 1, padded)
+template <int DT, int NSEG, int RD>
 __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 {
     constexpr int PS = NSEG + 1;      // pool segments of 64 slots per query
@@ -61,31 +71,21 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     float *ld = s_d[wv];
     int *li = s_i[wv];
 
-    const int K = a.K, D = a.D, nbd = a.nbd, ldc = a.ldc, nch = a.n_chunks;
+    const int K = a.K, nbd = a.nbd, ldc = a.ldc, nch = a.n_chunks;
     const float *__restrict__ sc = a.sc;
     const int *__restrict__ bb = a.bb;
-    const float *__restrict__ box_lo = a.box_lo;
-    const float *__restrict__ box_hi = a.box_hi;
 
     // ---- geometry (wave-uniform) ----
-    float mn[FGC_MAX_BIN_DIMS];
-    int nb[FGC_MAX_BIN_DIMS];
-#pragma unroll
-    for (int i = 0; i < FGC_MAX_BIN_DIMS; i++) {
-        mn[i] = a.geom[FGC_GEOM_MIN + i];
-        nb[i] = __float_as_int(a.geom[FGC_GEOM_NB + i]);
-    }
     const float bw = a.geom[FGC_GEOM_BW];
     const float margin = 1e-4f * bw;
-    int rnb[4];  // bins of the row dimensions (all binned dims but the last), padded with 1
+    int rnb[RD];  // bins of the row dimensions (all binned dimensions but the last), padded with 1
+    int rows_per_event = 1;
 #pragma unroll
-    for (int i = 0; i < 4; i++) rnb[i] = (i < nbd - 1) ? nb[i] : 1;
-    int nz = nb[0];
-    float mnz = mn[0];
-#pragma unroll
-    for (int i = 1; i < FGC_MAX_BIN_DIMS; i++)
-        if (i == nbd - 1) { nz = nb[i]; mnz = mn[i]; }
-    const int rows_per_event = rnb[0] * rnb[1] * rnb[2] * rnb[3];
+    for (int i = 0; i < RD; i++) {
+        rnb[i] = (i < nbd - 1) ? __float_as_int(a.geom[FGC_GEOM_NB + i]) : 1;
+        rows_per_event *= rnb[i];
+    }
+    const int nz = __float_as_int(a.geom[FGC_GEOM_NB + nbd - 1]);
 
     // ---- per-lane query state (lane q < nq holds query qbeg + q) ----
     const bool isq = lane < nq;
@@ -95,37 +95,35 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 #pragma unroll
         for (int d = 0; d < DR; d++) qx[d] = sc[(size_t)d * ldc + qs];
     }
-    float qb[4];  // normalised row-dimension coordinates
+    float qb[RD];  // normalised row-dimension coordinates
 #pragma unroll
-    for (int i = 0; i < 4; i++) qb[i] = (i < nbd - 1) ? sc[(size_t)i * ldc + qs] - mn[i] : 0.f;
-    const float qzn = sc[(size_t)(nbd - 1) * ldc + qs] - mnz;
-    const int key = (int)(a.skeys[qs] >> a.key_shift);
-    const int row = key / nz;
+    for (int i = 0; i < RD; i++) qb[i] = (i < nbd - 1) ? sc[(size_t)i * ldc + qs] - a.geom[FGC_GEOM_MIN + i] : 0.f;
+    const float qzn = sc[(size_t)(nbd - 1) * ldc + qs] - a.geom[FGC_GEOM_MIN + nbd - 1];
+    const int row = (int)(a.skeys[qs] >> a.key_shift) / nz;
     float tau = INFINITY;   // lane q: upper bound of query q's K-th distance
     int cnt = 0;            // lane q: candidates in query q's pool
     bool qactive = isq;
     if (a.sdir && isq) { unsigned char dd = a.sdir[qs]; qactive = !(dd == 0 || dd == 2); }
 
-    unsigned long long nev = 0, nchunks = 0, nins = 0, nevents = 0, ncullq = 0, nrows = 0, nqchunk = 0;
-
+    unsigned long long nev = 0;
+    unsigned nchunks = 0, nprunes = 0;
     const int slack = max(K >> 2, 4);   // a prune may keep up to K + slack candidates
 
     // ---- shrink query q's pool.  Finds a threshold t with at least K pool entries <= t by bisection
     //      (counts via wave ballots, the pool held one slot per lane and segment), keeps the entries
-    //      <= t and compacts them.  exact: t is the K-th smallest value itself and exactly K entries
-    //      stay (ties at t by slot order); otherwise a few bisection steps that stop as soon as at most
-    //      K + slack entries remain.  tau_q = t afterwards. ----
+    //      <= t and compacts them.  exact: exactly K entries stay (ties at the K-th value are cut by
+    //      slot order); otherwise the bisection stops as soon as at most K + slack entries remain.
+    //      tau_q = t afterwards. ----
     auto prune = [&](int q, bool exact) {
         const int c = fgc_readlane_i(cnt, q);
         if (c <= K) return;
         unsigned P[PS];
         int PI[PS];
-        bool valid[PS];
 #pragma unroll
         for (int s = 0; s < PS; s++) {
-            valid[s] = (s * 64 + lane) < c;
-            P[s] = valid[s] ? __float_as_uint(ld[q * CAP + s * 64 + lane]) : 0xffffffffu;
-            PI[s] = valid[s] ? li[q * CAP + s * 64 + lane] : -1;
+            const bool valid = (s * 64 + lane) < c;
+            P[s] = valid ? __float_as_uint(ld[q * CAP + s * 64 + lane]) : 0xffffffffu;
+            PI[s] = valid ? li[q * CAP + s * 64 + lane] : -1;
         }
         auto count_le = [&](unsigned t) -> int {
             int n = 0;
@@ -137,13 +135,16 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
         unsigned hi = (told < INFINITY) ? __float_as_uint(told) : 0x7f7fffffu;   // count_le(hi) >= K
         int chi = c;
         bool converged = false;
-        if (!exact && told < INFINITY) {
-            // linear bisection on [0, tau_old]; distances are non-negative floats
+        if (told < INFINITY) {
+            // linear bisection on [0, tau_old] (distances are non-negative); stops as soon as the count is
+            // inside [K, K + slack] - for an exact cut only at exactly K
+            const int accept = exact ? K : K + slack;
+            const int iters = exact ? 20 : 10;
             float flo = 0.f, fhi = told;
-            for (int it = 0; it < 10; it++) {
+            for (int it = 0; it < iters; it++) {
                 const float mid = 0.5f * (flo + fhi);
                 const int cm = count_le(__float_as_uint(mid));
-                if (cm >= K) { fhi = mid; chi = cm; if (cm <= K + slack) { converged = true; break; } }
+                if (cm >= K) { fhi = mid; chi = cm; if (cm <= accept) { converged = true; break; } }
                 else flo = mid;
             }
             hi = __float_as_uint(fhi);
@@ -155,7 +156,8 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             for (int s = 0; s < PS; s++) keep[s] = P[s] <= hi;
             newc = chi;
         } else {
-            // bisection on the bit pattern (monotone for non-negative floats) down to the K-th value itself
+            // bisection on the bit pattern (monotone for non-negative floats) down to the K-th value itself;
+            // ties at that value are cut by slot order
             unsigned lo = 0u;
             while (lo < hi) {
                 const unsigned mid = lo + ((hi - lo) >> 1);
@@ -184,131 +186,10 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             }
             base += __popcll(km);
         }
-        nins++;
+        nprunes++;
         const float tnew = __uint_as_float(hi);
         tau = (lane == q) ? tnew : tau;
         cnt = (lane == q) ? newc : cnt;
-    };
-
-    // ---- append the lanes of `pm` (distances dsq, sorted ids jbase + lane) to query q's pool ----
-    auto insert = [&](int q, unsigned long long pm, float dsq, int jbase) {
-        nevents++;
-        int c = fgc_readlane_i(cnt, q);
-        int np = __popcll(pm);
-        if (c + np > CAP) {
-            prune(q, false);
-            c = fgc_readlane_i(cnt, q);
-            pm = fgc_ballot(dsq < fgc_readlane_f(tau, q));
-            np = __popcll(pm);
-            if (c + np > CAP) {   // K + slack + a full chunk can exceed the pool: cut back to exactly K
-                prune(q, true);
-                c = fgc_readlane_i(cnt, q);
-                pm = fgc_ballot(dsq < fgc_readlane_f(tau, q));
-                np = __popcll(pm);
-            }
-            if (!pm) return;
-        }
-        if ((pm >> lane) & 1ull) {
-            const int pos = c + fgc_mbcnt(pm);
-            ld[q * CAP + pos] = dsq;
-            li[q * CAP + pos] = jbase + lane;
-        }
-        c += np;
-        cnt = (lane == q) ? c : cnt;
-        // keep tau tight: prune as soon as a quarter-chunk more than K candidates are pooled
-        if (c >= K + 32 || (c > K && !(fgc_readlane_f(tau, q) < INFINITY))) prune(q, false);
-    };
-
-    // ---- the candidates of chunk c inside [j0, j1) against the queries in `act` ----
-    auto process_chunk = [&](int c, int j0, int j1, unsigned long long act) {
-        const int base = c << 6;
-        const int j = base + lane;
-        const bool v = (j >= j0) && (j < j1);
-        float cx[DR];
-        if (DT > 0) {
-#pragma unroll
-            for (int d = 0; d < DR; d++) cx[d] = v ? sc[(size_t)d * ldc + j] : 0.f;
-        }
-        bool cand_ok = v;
-        if (a.sdir && v) { unsigned char dd = a.sdir[j]; if (dd == 1 || dd == 2) cand_ok = false; }
-        if (DT > 0 && !cand_ok) cx[0] = INFINITY;
-        nev += (unsigned long long)__popcll(act) * (unsigned)(min(j1, base + 64) - max(j0, base));
-        nchunks++;
-        nqchunk += __popcll(act);
-        unsigned long long m = act;
-        while (m) {
-            const int q = __ffsll((long long)m) - 1;
-            m &= m - 1;
-            const float t = fgc_readlane_f(tau, q);
-            float dsq;
-            if (DT > 0) {
-                float df = fgc_readlane_f(qx[0], q) - cx[0];
-                dsq = df * df;
-#pragma unroll
-                for (int d = 1; d < DR; d++) { df = fgc_readlane_f(qx[d], q) - cx[d]; dsq += df * df; }
-            } else {
-                dsq = INFINITY;
-                if (cand_ok) {
-                    float df = sc[qbeg + q] - sc[j];
-                    dsq = df * df;
-                    for (int d = 1; d < D; d++) {
-                        df = sc[(size_t)d * ldc + qbeg + q] - sc[(size_t)d * ldc + j];
-                        dsq += df * df;
-                    }
-                }
-            }
-            const unsigned long long pm = fgc_ballot(dsq < t);
-            if (pm) insert(q, pm, dsq, base);
-        }
-    };
-
-    // ---- all candidates in sorted positions [j0, j1) against the queries in `act`;
-    //      chunks seed_c0..seed_c1 were handled before and are skipped ----
-    auto process_span = [&](int j0, int j1, unsigned long long act, int seed_c0, int seed_c1) {
-        if (j0 >= j1 || !act) return;
-        const int c0 = j0 >> 6, c1 = (j1 - 1) >> 6;
-        if (DT == 0 || c1 - c0 + 1 < CULL_MIN) {
-            for (int c = c0; c <= c1; c++)
-                if (c < seed_c0 || c > seed_c1) process_chunk(c, j0, j1, act);
-            return;
-        }
-        // per-chunk bounding-box test, 64 chunks at a time (lane = chunk)
-        for (int cb = c0; cb <= c1; cb += 64) {
-            const int c = cb + lane;
-            const bool cv = (c <= c1) && (c < seed_c0 || c > seed_c1);
-            float blo[DR], bhi[DR];
-#pragma unroll
-            for (int d = 0; d < DR; d++) {
-                blo[d] = cv ? box_lo[(size_t)d * nch + c] : 0.f;
-                bhi[d] = cv ? box_hi[(size_t)d * nch + c] : 0.f;
-            }
-            unsigned mymask = 0;
-            unsigned long long m = act;
-            ncullq += __popcll(act);
-            while (m) {
-                const int q = __ffsll((long long)m) - 1;
-                m &= m - 1;
-                const float t = fgc_readlane_f(tau, q);
-                // same operation order as the distance: a candidate inside the box is never closer than this
-                float x = fgc_readlane_f(qx[0], q);
-                float g = fmaxf(fmaxf(blo[0] - x, x - bhi[0]), 0.f);
-                float g2 = g * g;
-#pragma unroll
-                for (int d = 1; d < DR; d++) {
-                    x = fgc_readlane_f(qx[d], q);
-                    g = fmaxf(fmaxf(blo[d] - x, x - bhi[d]), 0.f);
-                    g2 += g * g;
-                }
-                if (cv && !(g2 > t)) mymask |= 1u << q;
-            }
-            unsigned long long any = fgc_ballot(mymask != 0u);
-            while (any) {
-                const int l = __ffsll((long long)any) - 1;
-                any &= any - 1;
-                const unsigned long long cact = (unsigned long long)(unsigned)fgc_readlane_i((int)mymask, l);
-                process_chunk(cb + l, j0, j1, cact);
-            }
-        }
     };
 
     // squared gap (with safety margin) of this lane's query to a bin interval [b0, b1] of extent nbn
@@ -327,83 +208,215 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
         const unsigned long long gm = fgc_ballot(qactive && row == grow);
         todo &= ~gm;
         const int ev = grow / rows_per_event;
-        int rr = grow - ev * rows_per_event;
-        int c[4];
-        c[3] = rr % rnb[3]; rr /= rnb[3];
-        c[2] = rr % rnb[2]; rr /= rnb[2];
-        c[1] = rr % rnb[1]; rr /= rnb[1];
-        c[0] = rr;
+        int cr[RD];   // the group's own bin row
+        {
+            int rr = grow - ev * rows_per_event;
+#pragma unroll
+            for (int i = RD - 1; i >= 0; i--) { cr[i] = rr % rnb[i]; rr /= rnb[i]; }
+        }
         const int evrow0 = ev * rows_per_event;
         const int ev_j0 = bb[evrow0 * nz], ev_j1 = bb[(evrow0 + rows_per_event) * nz];
-
-        // -- seed: the chunks around the wavefront's own position, inside the event --
         const int own = qbeg >> 6;
         const int seed_c0 = max(own - NSEG, ev_j0 >> 6);
         const int seed_c1 = min(own + NSEG, (ev_j1 - 1) >> 6);
-        process_chunk(own, ev_j0, ev_j1, gm);
-        for (int cc = seed_c0; cc <= seed_c1; cc++)
-            if (cc != own) process_chunk(cc, ev_j0, ev_j1, gm);
 
-        // -- grow ring by ring over the bin rows --
-        for (int d = 0;; d++) {
-            // bins the balls of radius sqrt(tau) reach (whole grid while a query is not filled)
-            const bool filled = (fgc_ballot(tau < INFINITY) & gm) == gm;
-            int need_lo[4], need_hi[4], zlo = 0, zhi = nz - 1;
+        // span iteration state: phase 0 = own chunk, 1 = the other seed chunks, 2 = bin rows ring by ring
+        int phase = 0, d = 0;
+        int ai[RD], lo[RD], hi[RD];
+        int zlo = 0, zhi = nz - 1;
+        bool ring_open = false, ring_fresh = false, ring_any = false;
 #pragma unroll
-            for (int i = 0; i < 4; i++) { need_lo[i] = 0; need_hi[i] = rnb[i] - 1; }
-            if (filled) {
-                const float R = sqrtf(tau) * (1.0f + 1e-5f) + margin;
-                int blo[4], bhi[4];
+        for (int i = 0; i < RD; i++) { ai[i] = 0; lo[i] = 0; hi[i] = 0; }
+
+        for (;;) {
+            int j0, j1, sk0, sk1;
+            unsigned long long act;
+            if (phase == 0) {
+                j0 = max(ev_j0, own << 6); j1 = min(ev_j1, (own << 6) + 64);
+                sk0 = 1; sk1 = 0; act = gm; phase = 1;
+            } else if (phase == 1) {
+                j0 = max(ev_j0, seed_c0 << 6); j1 = min(ev_j1, (seed_c1 + 1) << 6);
+                sk0 = own; sk1 = own; act = gm; phase = 2;
+            } else {
+                if (!ring_open) {
+                    // start ring d: the bins the balls of radius sqrt(tau) reach (whole grid while a
+                    // query of the group has fewer than K candidates)
+                    const bool filled = (fgc_ballot(tau < INFINITY) & gm) == gm;
+                    int need_lo[RD], need_hi[RD];
+                    zlo = 0; zhi = nz - 1;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    blo[i] = (int)fminf(fmaxf(floorf((qb[i] - R) / bw + 1e-3f), 0.f), (float)(rnb[i] - 1));
-                    bhi[i] = (int)fminf(fmaxf(floorf((qb[i] + R) / bw + 1e-3f), 0.f), (float)(rnb[i] - 1));
-                    need_lo[i] = rnb[i] - 1;
-                    need_hi[i] = 0;
-                }
-                const int bzlo = (int)fminf(fmaxf(floorf((qzn - R) / bw + 1e-3f), 0.f), (float)(nz - 1));
-                const int bzhi = (int)fminf(fmaxf(floorf((qzn + R) / bw + 1e-3f), 0.f), (float)(nz - 1));
-                zlo = nz - 1;
-                zhi = 0;
-                for (unsigned long long mm = gm; mm;) {
-                    const int q = __ffsll((long long)mm) - 1;
-                    mm &= mm - 1;
+                    for (int i = 0; i < RD; i++) { need_lo[i] = 0; need_hi[i] = rnb[i] - 1; }
+                    if (filled) {
+                        const float R = sqrtf(tau) * (1.0f + 1e-5f) + margin;
+                        int blo[RD], bhi[RD];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        need_lo[i] = min(need_lo[i], fgc_readlane_i(blo[i], q));
-                        need_hi[i] = max(need_hi[i], fgc_readlane_i(bhi[i], q));
+                        for (int i = 0; i < RD; i++) {
+                            blo[i] = (int)fminf(fmaxf(floorf((qb[i] - R) / bw + 1e-3f), 0.f), (float)(rnb[i] - 1));
+                            bhi[i] = (int)fminf(fmaxf(floorf((qb[i] + R) / bw + 1e-3f), 0.f), (float)(rnb[i] - 1));
+                            need_lo[i] = rnb[i] - 1;
+                            need_hi[i] = 0;
+                        }
+                        const int bzlo = (int)fminf(fmaxf(floorf((qzn - R) / bw + 1e-3f), 0.f), (float)(nz - 1));
+                        const int bzhi = (int)fminf(fmaxf(floorf((qzn + R) / bw + 1e-3f), 0.f), (float)(nz - 1));
+                        zlo = nz - 1;
+                        zhi = 0;
+                        for (unsigned long long mm = gm; mm;) {
+                            const int q = __ffsll((long long)mm) - 1;
+                            mm &= mm - 1;
+#pragma unroll
+                            for (int i = 0; i < RD; i++) {
+                                need_lo[i] = min(need_lo[i], fgc_readlane_i(blo[i], q));
+                                need_hi[i] = max(need_hi[i], fgc_readlane_i(bhi[i], q));
+                            }
+                            zlo = min(zlo, fgc_readlane_i(bzlo, q));
+                            zhi = max(zhi, fgc_readlane_i(bzhi, q));
+                        }
                     }
-                    zlo = min(zlo, fgc_readlane_i(bzlo, q));
-                    zhi = max(zhi, fgc_readlane_i(bzhi, q));
+                    // rings 0..d-1 are done: stop when nothing outside them is needed
+                    bool done = d > 0;
+#pragma unroll
+                    for (int i = 0; i < RD; i++)
+                        done = done && (need_lo[i] >= cr[i] - (d - 1)) && (need_hi[i] <= cr[i] + (d - 1));
+                    if (done) break;
+#pragma unroll
+                    for (int i = 0; i < RD; i++) {
+                        lo[i] = max(cr[i] - d, 0);
+                        hi[i] = min(cr[i] + d, rnb[i] - 1);
+                        ai[i] = lo[i];
+                    }
+                    ring_open = true; ring_fresh = true; ring_any = false;
+                }
+                if (ring_fresh) {
+                    ring_fresh = false;
+                } else {
+                    bool carry = true;
+#pragma unroll
+                    for (int i = RD - 1; i >= 0; i--)
+                        if (carry) { if (ai[i] < hi[i]) { ai[i]++; carry = false; } else ai[i] = lo[i]; }
+                    if (carry) {             // ring finished
+                        ring_open = false;
+                        if (!ring_any) break;  // the ring lies outside the grid: everything has been visited
+                        d++;
+                        continue;
+                    }
+                }
+                int cheb = 0, rf = 0;
+                float g2 = gap1(qzn, zlo, zhi, nz);
+#pragma unroll
+                for (int i = 0; i < RD; i++) {
+                    cheb = max(cheb, abs(ai[i] - cr[i]));
+                    rf = rf * rnb[i] + ai[i];
+                    g2 += gap1(qb[i], ai[i], ai[i], rnb[i]);
+                }
+                if (cheb != d) continue;
+                ring_any = true;
+                act = gm & fgc_ballot(!(g2 > tau));
+                if (!act) continue;
+                const int b0 = (evrow0 + rf) * nz;
+                j0 = bb[b0 + zlo]; j1 = bb[b0 + zhi + 1];
+                sk0 = seed_c0; sk1 = seed_c1;
+            }
+            if (j0 >= j1) continue;
+
+            // ---- one span: sorted positions [j0, j1) against the queries in `act`, chunks sk0..sk1 skipped ----
+            const int c0 = j0 >> 6, c1 = (j1 - 1) >> 6;
+            const bool cull = (DT > 0) && (c1 - c0 + 1 >= CULL_MIN);
+            for (int cb = c0; cb <= c1; cb += 64) {
+                const int c = cb + lane;
+                const bool cv = (c <= c1) && (c < sk0 || c > sk1);
+                unsigned mymask = cv ? (unsigned)act : 0u;   // queries (bit q) that need chunk c
+                if (cull) {
+                    // per-chunk bounding-box test, lane = chunk
+                    float blo[DR], bhi[DR];
+#pragma unroll
+                    for (int dd = 0; dd < DR; dd++) {
+                        blo[dd] = cv ? a.box_lo[(size_t)dd * nch + c] : 0.f;
+                        bhi[dd] = cv ? a.box_hi[(size_t)dd * nch + c] : 0.f;
+                    }
+                    mymask = 0u;
+                    for (unsigned long long m = act; m;) {
+                        const int q = __ffsll((long long)m) - 1;
+                        m &= m - 1;
+                        const float t = fgc_readlane_f(tau, q);
+                        // same operation order as the distance: no candidate inside the box is closer than this
+                        float x = fgc_readlane_f(qx[0], q);
+                        float g = fmaxf(fmaxf(blo[0] - x, x - bhi[0]), 0.f);
+                        float g2 = g * g;
+#pragma unroll
+                        for (int dd = 1; dd < DR; dd++) {
+                            x = fgc_readlane_f(qx[dd], q);
+                            g = fmaxf(fmaxf(blo[dd] - x, x - bhi[dd]), 0.f);
+                            g2 += g * g;
+                        }
+                        if (cv && !(g2 > t)) mymask |= 1u << q;
+                    }
+                }
+                for (unsigned long long any = fgc_ballot(mymask != 0u); any;) {
+                    const int l = __ffsll((long long)any) - 1;
+                    any &= any - 1;
+                    const unsigned long long cact = (unsigned long long)(unsigned)fgc_readlane_i((int)mymask, l);
+                    // ---- chunk cb + l: one candidate per lane ----
+                    const int base = (cb + l) << 6;
+                    const int j = base + lane;
+                    const bool v = (j >= j0) && (j < j1);
+                    float cx[DR];
+                    if (DT > 0) {
+#pragma unroll
+                        for (int dd = 0; dd < DR; dd++) cx[dd] = v ? sc[(size_t)dd * ldc + j] : 0.f;
+                    }
+                    bool cand_ok = v;
+                    if (a.sdir && v) { unsigned char dd = a.sdir[j]; if (dd == 1 || dd == 2) cand_ok = false; }
+                    if (DT > 0 && !cand_ok) cx[0] = INFINITY;
+                    nev += (unsigned long long)__popcll(cact) * (unsigned)(min(j1, base + 64) - max(j0, base));
+                    nchunks++;
+                    for (unsigned long long m = cact; m;) {
+                        const int q = __ffsll((long long)m) - 1;
+                        m &= m - 1;
+                        const float t = fgc_readlane_f(tau, q);
+                        float dsq;
+                        if (DT > 0) {
+                            float df = fgc_readlane_f(qx[0], q) - cx[0];
+                            dsq = df * df;
+#pragma unroll
+                            for (int dd = 1; dd < DR; dd++) { df = fgc_readlane_f(qx[dd], q) - cx[dd]; dsq += df * df; }
+                        } else {
+                            dsq = INFINITY;
+                            if (cand_ok) {
+                                float df = sc[qbeg + q] - sc[j];
+                                dsq = df * df;
+                                for (int dd = 1; dd < a.D; dd++) {
+                                    df = sc[(size_t)dd * ldc + qbeg + q] - sc[(size_t)dd * ldc + j];
+                                    dsq += df * df;
+                                }
+                            }
+                        }
+                        unsigned long long pm = fgc_ballot(dsq < t);
+                        if (!pm) continue;
+                        // ---- append the passing lanes to query q's pool ----
+                        int pc = fgc_readlane_i(cnt, q);
+                        int np = __popcll(pm);
+#pragma nounroll
+                        for (int attempt = 0; attempt < 2 && pc + np > CAP; attempt++) {
+                            // make room: first a tighter threshold, then (K + slack + a full chunk can still
+                            // exceed the pool) a cut to exactly K
+                            prune(q, attempt == 1);
+                            pc = fgc_readlane_i(cnt, q);
+                            pm = fgc_ballot(dsq < fgc_readlane_f(tau, q));
+                            np = __popcll(pm);
+                        }
+                        if (!pm) continue;
+                        if ((pm >> lane) & 1ull) {
+                            const int pos = pc + fgc_mbcnt(pm);
+                            ld[q * CAP + pos] = dsq;
+                            li[q * CAP + pos] = j;
+                        }
+                        pc += np;
+                        cnt = (lane == q) ? pc : cnt;
+                        // keep tau tight: prune as soon as PRUNE_AT more than K candidates are pooled
+                        if (pc >= K + PRUNE_AT || (pc > K && !(t < INFINITY))) prune(q, false);
+                    }
                 }
             }
-            // rings 0..d-1 are done: stop when nothing outside them is needed
-            bool done = d > 0;
-#pragma unroll
-            for (int i = 0; i < 4; i++) done = done && (need_lo[i] >= c[i] - (d - 1)) && (need_hi[i] <= c[i] + (d - 1));
-            if (done) break;
-            int lo[4], hi[4];
-            bool any_row = false;
-#pragma unroll
-            for (int i = 0; i < 4; i++) { lo[i] = max(c[i] - d, 0); hi[i] = min(c[i] + d, rnb[i] - 1); }
-            for (int a0 = lo[0]; a0 <= hi[0]; a0++)
-                for (int a1 = lo[1]; a1 <= hi[1]; a1++)
-                    for (int a2 = lo[2]; a2 <= hi[2]; a2++)
-                        for (int a3 = lo[3]; a3 <= hi[3]; a3++) {
-                            const int cheb = max(max(abs(a0 - c[0]), abs(a1 - c[1])),
-                                                 max(abs(a2 - c[2]), abs(a3 - c[3])));
-                            if (cheb != d) continue;
-                            any_row = true;
-                            nrows++;
-                            const float g2 = gap1(qb[0], a0, a0, rnb[0]) + gap1(qb[1], a1, a1, rnb[1]) +
-                                             gap1(qb[2], a2, a2, rnb[2]) + gap1(qb[3], a3, a3, rnb[3]) +
-                                             gap1(qzn, zlo, zhi, nz);
-                            const unsigned long long act = gm & fgc_ballot(!(g2 > tau));
-                            if (!act) continue;
-                            const int b0 = (evrow0 + ((a0 * rnb[1] + a1) * rnb[2] + a2) * rnb[3] + a3) * nz;
-                            process_span(bb[b0 + zlo], bb[b0 + zhi + 1], act, seed_c0, seed_c1);
-                        }
-            if (!any_row) break;  // the ring lies outside the grid: everything has been visited
         }
     }
 
@@ -417,25 +430,46 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
         float L[NSEG];
         int I[NSEG], rank[NSEG];
         bool valid[NSEG];
+        bool has_self = false;
 #pragma unroll
         for (int s = 0; s < NSEG; s++) {
             valid[s] = (s * 64 + lane) < c;
             L[s] = valid[s] ? ld[q * CAP + s * 64 + lane] : INFINITY;
             I[s] = valid[s] ? li[q * CAP + s * 64 + lane] : -1;
-            if (valid[s] && I[s] == self) L[s] = -1.f;   // the query itself sorts first
+            const bool is_self = valid[s] && I[s] == self;
+            if (is_self) L[s] = -1.f;             // the query itself sorts first
+            has_self = has_self || (fgc_ballot(is_self) != 0ull);
             rank[s] = 0;
         }
-        bool has_self = false;
+        if (NSEG == 1) {
+            // bitonic sort of the 64 (distance, index) pairs across the lanes; equal keys never swap
+            float kd = L[0];
+            int kv = I[0];
 #pragma unroll
-        for (int s = 0; s < NSEG; s++) has_self = has_self || (fgc_ballot(valid[s] && I[s] == self) != 0ull);
-        // rank sort: position = number of entries that precede (by distance, then slot)
-        for (int e = 0; e < c; e++) {
-            float v = 0.f;
+            for (int k = 2; k <= 64; k <<= 1) {
 #pragma unroll
-            for (int s = 0; s < NSEG; s++)
-                if ((e >> 6) == s) v = fgc_readlane_f(L[s], e & 63);
+                for (int jj = k >> 1; jj > 0; jj >>= 1) {
+                    const float pd = __shfl_xor(kd, jj, 64);
+                    const int pv = __shfl_xor(kv, jj, 64);
+                    const bool keep_min = (((lane & jj) == 0) == ((lane & k) == 0));
+                    const bool take = keep_min ? (pd < kd) : (pd > kd);
+                    kd = take ? pd : kd;
+                    kv = take ? pv : kv;
+                }
+            }
+            L[0] = kd; I[0] = kv;
+            valid[0] = lane < c;                  // the c finite keys are now in lanes 0..c-1
+            rank[0] = lane;
+        } else {
+            // rank sort: position = number of entries that precede (by distance, then slot)
+            for (int e = 0; e < c; e++) {
+                float v = 0.f;
 #pragma unroll
-            for (int s = 0; s < NSEG; s++) rank[s] += ((v < L[s]) || (v == L[s] && e < s * 64 + lane)) ? 1 : 0;
+                for (int s = 0; s < NSEG; s++)
+                    if ((e >> 6) == s) v = fgc_readlane_f(L[s], e & 63);
+#pragma unroll
+                for (int s = 0; s < NSEG; s++) rank[s] += ((v < L[s]) || (v == L[s] && e < s * 64 + lane)) ? 1 : 0;
+            }
         }
         const int shift = has_self ? 0 : 1;       // without the query in the pool its slot 0 is added here
         const int n_out = min(c + shift, K);
@@ -460,37 +494,40 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     }
     if (a.stats && lane == 0) {
         atomicAdd(&a.stats[0], nev);
-        atomicAdd(&a.stats[1], nchunks);
-        atomicAdd(&a.stats[2], nins);
-        atomicAdd(&a.stats[3], nevents);
-        atomicAdd(&a.stats[4], ncullq);
-        atomicAdd(&a.stats[5], nrows);
-        atomicAdd(&a.stats[6], nqchunk);
+        atomicAdd(&a.stats[1], (unsigned long long)nchunks);
+        atomicAdd(&a.stats[2], (unsigned long long)nprunes);
     }
 }
 
-template <int DT, int NSEG> static int launch_knn_t(const KnnArgs &a, hipStream_t s)
+template <int DT, int NSEG, int RD> static int launch_knn_t(const KnnArgs &a, hipStream_t s)
 {
     constexpr int WPB = KnnCfg<NSEG>::WPB;
     const int tiles = (int)fgc_cdiv(a.n, QT);
     const int blocks = (int)fgc_cdiv(tiles, WPB);
-    hipLaunchKernelGGL((k_knn<DT, NSEG>), dim3(blocks), dim3(WPB * 64), 0, s, a);
+    hipLaunchKernelGGL((k_knn<DT, NSEG, RD>), dim3(blocks), dim3(WPB * 64), 0, s, a);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
 
-template <int NSEG> static int launch_knn_d(const KnnArgs &a, hipStream_t s)
+template <int NSEG, int RD> static int launch_knn_d(const KnnArgs &a, hipStream_t s)
 {
     switch (a.D) {
-    case 2: return launch_knn_t<2, NSEG>(a, s);
-    case 3: return launch_knn_t<3, NSEG>(a, s);
-    case 4: return launch_knn_t<4, NSEG>(a, s);
-    case 5: return launch_knn_t<5, NSEG>(a, s);
-    case 6: return launch_knn_t<6, NSEG>(a, s);
-    case 7: return launch_knn_t<7, NSEG>(a, s);
-    case 8: return launch_knn_t<8, NSEG>(a, s);
-    default: return launch_knn_t<0, NSEG>(a, s);
+    case 2: return launch_knn_t<2, NSEG, RD>(a, s);
+    case 3: return launch_knn_t<3, NSEG, RD>(a, s);
+    case 4: return launch_knn_t<4, NSEG, RD>(a, s);
+    case 5: return launch_knn_t<5, NSEG, RD>(a, s);
+    case 6: return launch_knn_t<6, NSEG, RD>(a, s);
+    case 7: return launch_knn_t<7, NSEG, RD>(a, s);
+    case 8: return launch_knn_t<8, NSEG, RD>(a, s);
+    default: return launch_knn_t<0, NSEG, RD>(a, s);
     }
+}
+
+template <int NSEG> static int launch_knn_r(const KnnArgs &a, hipStream_t s)
+{
+    if (a.nbd <= 2) return launch_knn_d<NSEG, 1>(a, s);
+    if (a.nbd == 3) return launch_knn_d<NSEG, 2>(a, s);
+    return launch_knn_d<NSEG, 4>(a, s);
 }
 
 int fgc_launch_knn(const KnnArgs &a, hipStream_t s)
@@ -498,7 +535,7 @@ int fgc_launch_knn(const KnnArgs &a, hipStream_t s)
     if (a.n <= 0) return FGC_OK;
     if (a.K < 1 || a.K > FGC_MAX_K || a.D < 1 || a.nbd < 1 || a.nbd > FGC_MAX_BIN_DIMS || a.nbd > a.D)
         return FGC_EINVAL;
-    if (a.K <= 64) return launch_knn_d<1>(a, s);
-    if (a.K <= 128) return launch_knn_d<2>(a, s);
-    return launch_knn_d<4>(a, s);
+    if (a.K <= 64) return launch_knn_r<1>(a, s);
+    if (a.K <= 128) return launch_knn_r<2>(a, s);
+    return launch_knn_r<4>(a, s);
 }
