@@ -20,6 +20,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
+# HBM bytes per k_knn launch at the default workload, from two rocprofv3 --pmc runs (FETCH_SIZE x 1.99 KiB
+# + WRITE_SIZE x 1.00 KiB, factors from a plain copy kernel in the same runs)
+KNN_TRAFFIC_CFG4_BYTES = 960.6e6
 
 
 def main():
@@ -132,7 +135,8 @@ def main():
     bytes_alg = 4.0 * D * c_eval + 4.0 * D * n + 12.0 * K * n
     achieved = bytes_alg / (t_knn * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "k_knn", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": KNN_TRAFFIC_CFG4_BYTES if (args.workload == "cfg4" and args.scale == 1.0) else None,
                 "algorithmic_bytes": bytes_alg, "distance_evaluations": c_eval,
                 "kernel_ms": round(t_knn, 4), "io_floor_bytes": 4.0 * D * n + 12.0 * K * n}
 

@@ -46,7 +46,9 @@
 #ifndef PRUNE_AT
 #define PRUNE_AT 32    // a pool is pruned when it holds this many candidates more than K
 #endif
+#ifndef CULL_MIN
 #define CULL_MIN 3     // spans of at least this many chunks get the per-chunk box test
+#endif
 
 // wavefronts per block, chosen so that a block's pools fit the 64 KB static LDS limit
 template <int NSEG> struct KnnCfg { static constexpr int WPB = (NSEG <= 2 ? 2 : 1) * (16 / QT); };
