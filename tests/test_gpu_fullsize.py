@@ -1,0 +1,117 @@
+"""The benchmark configurations at their full sizes on the GPU: size-independent
+invariants, exhaustive-search checks on sampled queries, and full comparisons
+with the CPU checker where that takes seconds."""
+import numpy as np
+import pytest
+import torch
+
+from tests.util import assert_knn_equal, check_knn_properties, DIST_RTOL
+
+pytestmark = pytest.mark.gpu
+
+
+def _brute_rows(coords, rs, queries, K):
+    """float32 exhaustive search for the given query rows, same operation order as the kernels."""
+    rs = np.asarray(rs)
+    out_d = np.zeros((len(queries), K), np.float32)
+    out_i = np.full((len(queries), K), -1, np.int64)
+    for r, i in enumerate(queries):
+        e = np.searchsorted(rs[1:], i, side="right")
+        a, b = int(rs[e]), int(rs[e + 1])
+        diff = coords[a:b] - coords[i]
+        d2 = diff[:, 0] * diff[:, 0]
+        for c in range(1, coords.shape[1]):
+            d2 = d2 + diff[:, c] * diff[:, c]
+        d2[i - a] = -1.0                      # the query itself first
+        kk = min(K, b - a)
+        part = np.argpartition(d2, kk - 1)[:kk]
+        part = part[np.lexsort((part, d2[part]))]
+        out_i[r, :kk] = part + a
+        out_d[r, :kk] = np.maximum(d2[part], 0.0)
+    return out_i, out_d
+
+
+def _run(w):
+    from fastgraphcompute_amd import binned_select_knn
+    idx, dist = binned_select_knn(w["K"], torch.from_numpy(w["coords"]).cuda(),
+                                  torch.from_numpy(w["row_splits"]).cuda())
+    return idx.cpu().numpy(), dist.cpu().numpy()
+
+
+def _sample_check(w, gi, gd, n_samples, seed):
+    rng = np.random.default_rng(seed)
+    q = np.sort(rng.choice(w["coords"].shape[0], n_samples, replace=False))
+    bi, bd = _brute_rows(w["coords"], w["row_splits"], q, w["K"])
+    assert_knn_equal(gi[q], gd[q], bi, bd, "sampled exhaustive search")
+
+
+def test_cfg4_full_forward_and_gradient(oracle):
+    from fastgraphcompute_amd.workloads import cfg4_zipf_blobs
+    from fastgraphcompute_amd.extensions import binned_select_knn_grad
+    w = cfg4_zipf_blobs()
+    gi, gd = _run(w)
+    check_knn_properties(gi, gd, w["coords"], w["row_splits"], w["K"])
+    _sample_check(w, gi, gd, 300, 4)
+    # densest region: the queries with the smallest K-th distance
+    dense = np.argsort(gd[:, -1])[:100]
+    bi, bd = _brute_rows(w["coords"], w["row_splits"], np.sort(dense), w["K"])
+    assert_knn_equal(gi[np.sort(dense)], gd[np.sort(dense)], bi, bd, "densest queries")
+    # gradient: full comparison with the checker, plus translation invariance (the gradients sum to zero)
+    x = torch.from_numpy(w["coords"]).cuda()
+    it = torch.from_numpy(gi).cuda()
+    g1 = torch.from_numpy(w["grad_distsq"]).cuda()
+    got = binned_select_knn_grad(g1, it, x).cpu().numpy()
+    exp = oracle.knn_grad(w["grad_distsq"], gi, w["coords"])
+    scale = np.abs(exp).max()
+    assert np.abs(got - exp).max() <= DIST_RTOL * scale
+    assert np.abs(got.astype(np.float64).sum(axis=0)).max() <= 1e-3 * scale
+    # linearity in the upstream gradient
+    g2 = torch.from_numpy(np.random.default_rng(5).standard_normal(g1.shape).astype(np.float32)).cuda()
+    lin = binned_select_knn_grad(2.0 * g1 - 0.5 * g2, it, x).cpu().numpy()
+    sep = 2.0 * got - 0.5 * binned_select_knn_grad(g2, it, x).cpu().numpy()
+    assert np.abs(lin - sep).max() <= 2 * DIST_RTOL * np.abs(sep).max()
+
+
+def test_cfg2_full_against_checker(oracle):
+    from fastgraphcompute_amd.workloads import cfg2_blobs_4events
+    w = cfg2_blobs_4events()
+    gi, gd = _run(w)
+    check_knn_properties(gi, gd, w["coords"], w["row_splits"], w["K"])
+    oi, od = oracle.binned_select_knn(w["K"], w["coords"], w["row_splits"], n_threads=16)
+    assert_knn_equal(gi, gd, oi, od)
+
+
+def test_cfg5_full_sampled(oracle):
+    from fastgraphcompute_amd.workloads import cfg5_many_events_d8
+    w = cfg5_many_events_d8()
+    gi, gd = _run(w)
+    check_knn_properties(gi, gd, w["coords"], w["row_splits"], w["K"])
+    _sample_check(w, gi, gd, 400, 6)
+
+
+def test_cfg3_gravnet_full(oracle):
+    from fastgraphcompute_amd.workloads import cfg3_gravnet
+    from fastgraphcompute_amd.gnn_ops import GravNetOp, gravnet_aggregate
+    w = cfg3_gravnet()
+    torch.manual_seed(w["weight_seed"])
+    op = GravNetOp(w["in_channels"], w["out_channels"], w["space_dimensions"], w["propagate_dimensions"], w["K"]).cuda()
+    x = torch.from_numpy(w["x"]).cuda().requires_grad_(True)
+    rs = torch.from_numpy(w["row_splits"]).cuda()
+    out, idx, dsq, space = op(x, rs)
+    (out * torch.from_numpy(w["out_grad"]).cuda()).sum().backward()
+    n = w["x"].shape[0]
+    assert out.shape == (n, 64) and idx.shape == (n, 40) and space.shape == (n, 4)
+    assert torch.isfinite(out).all() and torch.isfinite(x.grad).all()
+    for p in op.parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all()
+    ih, dh, sh = idx.cpu().numpy(), dsq.detach().cpu().numpy(), space.detach().cpu().numpy()
+    check_knn_properties(ih, dh, sh, w["row_splits"], 40)
+    q = np.sort(np.random.default_rng(7).choice(n, 200, replace=False))
+    bi, bd = _brute_rows(sh, w["row_splits"], q, 40)
+    assert_knn_equal(ih[q], dh[q], bi, bd, "GravNet learned space")
+    # the fused aggregation on the full tensors against the checker's kernel
+    prop = op.propagate_transformations(x).detach()
+    fm, fx = gravnet_aggregate(idx, dsq.detach(), prop)
+    cm, cx, _ = oracle.gravnet_aggregate(ih, dh, prop.cpu().numpy())
+    assert np.abs(fm.cpu().numpy() - cm).max() <= DIST_RTOL * np.abs(cm).max()
+    assert np.abs(fx.cpu().numpy() - cx).max() <= DIST_RTOL * np.abs(cx).max()
