@@ -30,7 +30,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg4", "cfg5"])
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seconds", type=float, default=15.0)
@@ -55,6 +55,8 @@ def main():
     L = _lib.lib()
 
     w = workloads.CONFIGS[args.workload](args.scale)
+    if args.workload == "cfg3":
+        return gravnet_workload(args, w, dev)
     K = int(w["K"])
     coords_h = w["coords"]
     n, D = coords_h.shape
@@ -159,6 +161,39 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, K, n, args.cpu_sample_seconds)
     print(json.dumps(result), flush=True)
+
+
+def gravnet_workload(args, w, dev):
+    """Secondary workload: one GravNetOp forward + backward (N = 300 000 x 64 features, S=4, P=32, k=40)."""
+    import torch
+    from fastgraphcompute_amd.gnn_ops import GravNetOp
+    torch.manual_seed(w["weight_seed"])
+    op = GravNetOp(w["in_channels"], w["out_channels"], w["space_dimensions"], w["propagate_dimensions"],
+                   w["K"]).to(dev)
+    x = torch.from_numpy(w["x"]).to(dev).requires_grad_(True)
+    rs = torch.from_numpy(w["row_splits"]).to(dev)
+    g = torch.from_numpy(w["out_grad"]).to(dev)
+
+    def step():
+        x.grad = None
+        op.zero_grad(set_to_none=True)
+        out = op(x, rs)[0]
+        out.backward(g)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / args.steps
+    n = w["x"].shape[0]
+    print(json.dumps({
+        "metric": "GravNetOp forward+backward points/sec", "value": round(n / t, 1), "unit": "points/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(t * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": w["name"], "n_points": n, "events": 2}}), flush=True)
 
 
 def cpu_baseline(w, K, n, budget_s):
