@@ -30,6 +30,7 @@ struct KnnArgs {
     int nbd;                    // binned dimensions
     int K;
     int tf_compat;
+    int pool_cap;               // candidate pool slots per query (set by fgc_launch_knn)
     int64_t *out_idx;           // [n, K] original order
     float *out_dist;            // [n, K]
     unsigned long long *stats;  // optional counters

@@ -43,8 +43,11 @@
 #ifndef QT
 #define QT 8           // queries per wavefront
 #endif
-#ifndef PRUNE_AT
-#define PRUNE_AT 32    // a pool is pruned when it holds this many candidates more than K
+#ifndef POOL_EXTRA
+#define POOL_EXTRA 48  // pool slots beyond K (rounded up to 16); LDS per wavefront = QT * pool slots * 8 B
+#endif
+#ifndef PRUNE_MARGIN
+#define PRUNE_MARGIN 8 // a pool is pruned when fewer than this many slots are free
 #endif
 #ifndef CULL_MIN
 #define CULL_MIN 3     // spans of at least this many chunks get the per-chunk box test
@@ -58,20 +61,19 @@ template <int NSEG> struct KnnCfg { static constexpr int WPB = (NSEG <= 2 ? 2 : 
 template <int DT, int NSEG, int RD>
 __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 {
-    constexpr int PS = NSEG + 1;      // pool segments of 64 slots per query
-    constexpr int CAP = PS * 64;      // pool capacity: K kept + one chunk of new candidates
+    constexpr int PS = NSEG + 1;          // pool segments (lanes x PS cover the pool)
     constexpr int WPB = KnnCfg<NSEG>::WPB;
     constexpr int DR = DT > 0 ? DT : 1;
-    __shared__ float s_d[WPB][QT * CAP];
-    __shared__ int s_i[WPB][QT * CAP];
+    extern __shared__ float s_pool[];     // [WPB][2][QT * CAP]: distances, then sorted positions (as int)
+    const int CAP = a.pool_cap;           // pool capacity per query: K kept + room for new candidates
 
     const int lane = fgc_lane();
     const int wv = threadIdx.x >> 6;
     const int qbeg = (blockIdx.x * WPB + wv) * QT;
     if (qbeg >= a.n) return;  // no block-wide barrier is used below
     const int nq = min(QT, a.n - qbeg);
-    float *ld = s_d[wv];
-    int *li = s_i[wv];
+    float *ld = s_pool + (size_t)wv * 2 * QT * CAP;
+    int *li = (int *)(ld + QT * CAP);
 
     const int K = a.K, nbd = a.nbd, ldc = a.ldc, nch = a.n_chunks;
     const float *__restrict__ sc = a.sc;
@@ -394,28 +396,43 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                         }
                         unsigned long long pm = fgc_ballot(dsq < t);
                         if (!pm) continue;
-                        // ---- append the passing lanes to query q's pool ----
+                        // ---- append the passing lanes to query q's pool, pruning when it runs full: first to
+                        //      a tighter threshold, then (if that is not enough) down to exactly K ----
                         int pc = fgc_readlane_i(cnt, q);
-                        int np = __popcll(pm);
-#pragma nounroll
-                        for (int attempt = 0; attempt < 2 && pc + np > CAP; attempt++) {
-                            // make room: first a tighter threshold, then (K + slack + a full chunk can still
-                            // exceed the pool) a cut to exactly K
-                            prune(q, attempt == 1);
-                            pc = fgc_readlane_i(cnt, q);
-                            pm = fgc_ballot(dsq < fgc_readlane_f(tau, q));
-                            np = __popcll(pm);
+                        if (__popcll(pm) <= CAP - pc) {
+                            if ((pm >> lane) & 1ull) {
+                                const int pos = pc + fgc_mbcnt(pm);
+                                ld[q * CAP + pos] = dsq;
+                                li[q * CAP + pos] = j;
+                            }
+                            pc += __popcll(pm);
+                            cnt = (lane == q) ? pc : cnt;
+                        } else {
+                            int attempt = 0;
+                            while (pm) {
+                                int room = CAP - pc;
+                                if (__popcll(pm) > room) {
+                                    prune(q, attempt > 0);
+                                    attempt++;
+                                    pm &= fgc_ballot(dsq < fgc_readlane_f(tau, q));
+                                    pc = fgc_readlane_i(cnt, q);
+                                    room = CAP - pc;
+                                    if (!pm) break;
+                                }
+                                const int rnk = fgc_mbcnt(pm);
+                                const bool put = ((pm >> lane) & 1ull) && rnk < room;
+                                const unsigned long long sub = fgc_ballot(put);
+                                if (put) {
+                                    ld[q * CAP + pc + rnk] = dsq;
+                                    li[q * CAP + pc + rnk] = j;
+                                }
+                                pc += __popcll(sub);
+                                cnt = (lane == q) ? pc : cnt;
+                                pm &= ~sub;
+                            }
                         }
-                        if (!pm) continue;
-                        if ((pm >> lane) & 1ull) {
-                            const int pos = pc + fgc_mbcnt(pm);
-                            ld[q * CAP + pos] = dsq;
-                            li[q * CAP + pos] = j;
-                        }
-                        pc += np;
-                        cnt = (lane == q) ? pc : cnt;
-                        // keep tau tight: prune as soon as PRUNE_AT more than K candidates are pooled
-                        if (pc >= K + PRUNE_AT || (pc > K && !(t < INFINITY))) prune(q, false);
+                        // keep tau tight: prune as soon as the pool is nearly full
+                        if (pc > CAP - PRUNE_MARGIN || (pc > K && !(fgc_readlane_f(tau, q) < INFINITY))) prune(q, false);
                     }
                 }
             }
@@ -506,7 +523,8 @@ template <int DT, int NSEG, int RD> static int launch_knn_t(const KnnArgs &a, hi
     constexpr int WPB = KnnCfg<NSEG>::WPB;
     const int tiles = (int)fgc_cdiv(a.n, QT);
     const int blocks = (int)fgc_cdiv(tiles, WPB);
-    hipLaunchKernelGGL((k_knn<DT, NSEG, RD>), dim3(blocks), dim3(WPB * 64), 0, s, a);
+    const size_t lds = (size_t)WPB * 2 * QT * a.pool_cap * sizeof(float);
+    hipLaunchKernelGGL((k_knn<DT, NSEG, RD>), dim3(blocks), dim3(WPB * 64), lds, s, a);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
@@ -532,11 +550,13 @@ template <int NSEG> static int launch_knn_r(const KnnArgs &a, hipStream_t s)
     return launch_knn_d<NSEG, 4>(a, s);
 }
 
-int fgc_launch_knn(const KnnArgs &a, hipStream_t s)
+int fgc_launch_knn(const KnnArgs &a_in, hipStream_t s)
 {
+    KnnArgs a = a_in;
     if (a.n <= 0) return FGC_OK;
     if (a.K < 1 || a.K > FGC_MAX_K || a.D < 1 || a.nbd < 1 || a.nbd > FGC_MAX_BIN_DIMS || a.nbd > a.D)
         return FGC_EINVAL;
+    a.pool_cap = ((a.K + POOL_EXTRA + 15) / 16) * 16;   // <= 64 * (ceil(K / 64) + 1)
     if (a.K <= 64) return launch_knn_r<1>(a, s);
     if (a.K <= 128) return launch_knn_r<2>(a, s);
     return launch_knn_r<4>(a, s);

@@ -37,7 +37,12 @@ extern "C" int fgc_index_replacer_i64(const int64_t *d_in, const int64_t *d_repl
 // table (open addressing, LDS float atomics); only the distinct targets go to
 // global memory, one float atomic per coordinate.  Pairs that find no slot
 // within a few probes go to global memory directly.
-#define GQ 64          // queries per block (4 wavefronts x 16)
+#ifndef GQ
+#define GQ 64          // queries per block (4 wavefronts x GQ/4)
+#endif
+#ifndef GRAD_H
+#define GRAD_H 2048     // hash table slots per block (upper bound, shrunk for wide points)
+#endif
 #define GRAD_PROBES 8
 #define GRAD_EMPTY 0xffffffffu
 
@@ -103,21 +108,21 @@ __global__ __launch_bounds__(256) void k_knn_grad(const float *__restrict__ gd, 
         }
     }
     __syncthreads();
-    for (int t = threadIdx.x; t < H; t += 256) {
-        const unsigned m = keys[t];
+    // one lane per (slot, coordinate): the atomics of one target sit in adjacent lanes
+    for (int t = threadIdx.x; t < H * D; t += 256) {
+        const int sl = t / D;
+        const unsigned m = keys[sl];
         if (m == GRAD_EMPTY) continue;
-        for (int c = 0; c < D; c++) {
-            const float v = vals[t * D + c];
-            if (v != 0.f) atomicAdd(&gx[(int64_t)m * D + c], v);
-        }
+        const float v = vals[t];
+        if (v != 0.f) atomicAdd(&gx[(int64_t)m * D + (t - sl * D)], v);
     }
     if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
 }
 
 static int grad_table_size(int D)
 {
-    int H = 2048;
-    while (H > 64 && (size_t)H * (4 + 4 * (size_t)D) > 40960) H >>= 1;
+    int H = GRAD_H;
+    while (H > 64 && (size_t)H * (4 + 4 * (size_t)D) > 65536) H >>= 1;
     return H;
 }
 
