@@ -373,52 +373,62 @@ __global__ __launch_bounds__(256) void k_rs_hist(const uint32_t *__restrict__ ke
     block_hist[threadIdx.x * nblk + blockIdx.x] = s_h[threadIdx.x];
 }
 
-// in-place exclusive scan of `len` uint32 values by one 1024-thread block,
-// in coalesced tiles of 8192 values (8 consecutive values per thread);
-// if total != NULL it receives the sum
-__global__ __launch_bounds__(1024) void k_scan_excl_u32(uint32_t *__restrict__ a, int len,
-                                                        uint32_t *__restrict__ total)
+// exclusive scan of every digit's row of per-block counts (one block per digit, in place);
+// digit_total[digit] receives the row sum
+__global__ __launch_bounds__(256) void k_rs_scan_rows(uint32_t *__restrict__ block_hist, int nblk,
+                                                      uint32_t *__restrict__ digit_total)
 {
-    __shared__ uint32_t s_w[16];
+    __shared__ uint32_t s_w[4];
     __shared__ uint32_t s_carry;
+    uint32_t *row = block_hist + (size_t)blockIdx.x * nblk;
     const int t = threadIdx.x, lane = t & 63, wv = t >> 6;
     if (t == 0) s_carry = 0;
     __syncthreads();
-    for (int base = 0; base < len; base += 8192) {
-        const int i0 = base + t * 8;
-        uint32_t v[8];
-        uint32_t sum = 0;
-#pragma unroll
-        for (int k = 0; k < 8; k++) { v[k] = (i0 + k < len) ? a[i0 + k] : 0u; sum += v[k]; }
-        uint32_t incl = sum;
+    for (int base = 0; base < nblk; base += 256) {
+        const int i = base + t;
+        const uint32_t v = (i < nblk) ? row[i] : 0u;
+        uint32_t incl = v;
         for (int o = 1; o < 64; o <<= 1) {
             uint32_t u = __shfl_up(incl, o, 64);
             if (lane >= o) incl += u;
         }
         if (lane == 63) s_w[wv] = incl;
         __syncthreads();
-        uint32_t woff = s_carry;
-        for (int w = 0; w < wv; w++) woff += s_w[w];
-        uint32_t run = woff + incl - sum;
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            if (i0 + k < len) a[i0 + k] = run;
-            run += v[k];
-        }
+        uint32_t off = s_carry;
+        for (int w = 0; w < wv; w++) off += s_w[w];
+        if (i < nblk) row[i] = off + incl - v;
         __syncthreads();
-        if (t == 1023) s_carry = run;
+        if (t == 255) s_carry = off + incl;
         __syncthreads();
     }
-    if (total && t == 0) *total = s_carry;
+    if (t == 0) digit_total[blockIdx.x] = s_carry;
 }
 
 __global__ __launch_bounds__(256) void k_rs_scatter(const uint32_t *__restrict__ keys_in,
                                                     const uint32_t *__restrict__ vals_in,
                                                     uint32_t *__restrict__ keys_out,
                                                     uint32_t *__restrict__ vals_out, int n, int shift,
-                                                    int nblk, const uint32_t *__restrict__ block_hist)
+                                                    int nblk, const uint32_t *__restrict__ block_hist,
+                                                    const uint32_t *__restrict__ digit_total)
 {
     __shared__ uint32_t s_cnt[4][256];
+    __shared__ uint32_t s_dig[256];   // exclusive scan of the digit totals
+    {
+        __shared__ uint32_t s_ws[4];
+        const int t = threadIdx.x, ln = t & 63, w = t >> 6;
+        const uint32_t v = digit_total[t];
+        uint32_t incl = v;
+        for (int o = 1; o < 64; o <<= 1) {
+            uint32_t u = __shfl_up(incl, o, 64);
+            if (ln >= o) incl += u;
+        }
+        if (ln == 63) s_ws[w] = incl;
+        __syncthreads();
+        uint32_t off = 0;
+        for (int k = 0; k < w; k++) off += s_ws[k];
+        s_dig[t] = off + incl - v;
+        __syncthreads();
+    }
     const int lane = fgc_lane(), wv = threadIdx.x >> 6;
     volatile uint32_t *cnt = s_cnt[wv];
     for (int i = lane; i < 256; i += 64) cnt[i] = 0;
@@ -438,7 +448,7 @@ __global__ __launch_bounds__(256) void k_rs_scatter(const uint32_t *__restrict__
     // per-digit exclusive offsets of the four waves on top of the global base
     {
         int t = threadIdx.x;
-        uint32_t g = block_hist[t * nblk + blockIdx.x];
+        uint32_t g = s_dig[t] + block_hist[t * nblk + blockIdx.x];
         for (int w = 0; w < 4; w++) {
             uint32_t c = s_cnt[w][t];
             s_cnt[w][t] = g;
@@ -467,7 +477,8 @@ __global__ __launch_bounds__(256) void k_rs_scatter(const uint32_t *__restrict__
 size_t fgc_sort_workspace_bytes(int64_t n)
 {
     int64_t nblk = fgc_cdiv(n > 0 ? n : 1, RS_TILE);
-    return fgc_align((size_t)n * 4) * 2 /* ping-pong keys / vals */ + fgc_align((size_t)nblk * 256 * 4);
+    return fgc_align((size_t)n * 4) * 2 /* ping-pong keys / vals */ + fgc_align((size_t)nblk * 256 * 4) +
+           fgc_align(256 * 4) /* digit totals */;
 }
 
 // Sorts (keys, identity) stably by the low `key_bits` bits.  On return
@@ -482,6 +493,7 @@ int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void 
     uint32_t *v_alt = (uint32_t *)w; w += fgc_align((size_t)n * 4);
     uint32_t *hist = (uint32_t *)w;
     int nblk = (int)fgc_cdiv(n, RS_TILE);
+    uint32_t *digit_total = (uint32_t *)(w + fgc_align((size_t)nblk * 256 * 4));
     if ((int64_t)nblk * 256 >= (1ll << 31)) return FGC_EINVAL;
     uint32_t *kin = keys, *vin = nullptr, *kout = k_alt, *vout = v_alt;
     int passes = (key_bits + 7) / 8;
@@ -490,10 +502,10 @@ int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void 
         int shift = p * 8;
         hipLaunchKernelGGL(k_rs_hist, dim3(nblk), dim3(256), 0, s, kin, (int)n, shift, nblk, hist);
         FGC_LAUNCH_CHECK();
-        hipLaunchKernelGGL(k_scan_excl_u32, dim3(1), dim3(1024), 0, s, hist, nblk * 256, (uint32_t *)nullptr);
+        hipLaunchKernelGGL(k_rs_scan_rows, dim3(256), dim3(256), 0, s, hist, nblk, digit_total);
         FGC_LAUNCH_CHECK();
         hipLaunchKernelGGL(k_rs_scatter, dim3(nblk), dim3(256), 0, s, kin, vin, kout, vout, (int)n, shift,
-                           nblk, hist);
+                           nblk, hist, digit_total);
         FGC_LAUNCH_CHECK();
         kin = kout; vin = vout;
         if (kout == k_alt) { kout = keys; vout = vals; } else { kout = k_alt; vout = v_alt; }

@@ -99,6 +99,7 @@ class _BinnedKNN(torch.autograd.Function):
             order = torch.empty(0, dtype=torch.int32, device=dev)
         ctx.save_for_backward(idx, coords, order)
         ctx.mark_non_differentiable(idx)
+        ctx.set_materialize_grads(False)   # no zero tensors for unused output gradients
         return idx, dist
 
     @staticmethod

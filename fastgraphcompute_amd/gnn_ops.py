@@ -29,6 +29,7 @@ class _GravNetAggregate(torch.autograd.Function):
             _lib.check(L.fgc_gravnet_aggregate_fwd_f32(_lib.ptr(ii), _lib.ptr(d), _lib.ptr(f), _lib.ptr(fmean),
                                                        _lib.ptr(fmax), _lib.ptr(argmax), n, K, P, _lib.stream_ptr()))
         ctx.save_for_backward(ii, d, f, argmax)
+        ctx.set_materialize_grads(False)
         return fmean, fmax
 
     @staticmethod
@@ -37,8 +38,12 @@ class _GravNetAggregate(torch.autograd.Function):
         L = _lib.lib()
         n, K = ii.shape
         P = f.shape[1]
-        g_mean = torch.zeros_like(f[:n]) if g_mean is None else g_mean.to(torch.float32).contiguous()
-        g_max = torch.zeros_like(f[:n]) if g_max is None else g_max.to(torch.float32).contiguous()
+        if g_mean is None and g_max is None:
+            return None, None, None
+        g_mean = torch.zeros((n, P), dtype=torch.float32, device=f.device) if g_mean is None \
+            else g_mean.to(torch.float32).contiguous()
+        g_max = torch.zeros((n, P), dtype=torch.float32, device=f.device) if g_max is None \
+            else g_max.to(torch.float32).contiguous()
         g_feat = torch.zeros_like(f)
         g_dist = torch.empty_like(d)
         with torch.cuda.device(f.device):
