@@ -68,7 +68,9 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     const int CAP = a.pool_cap;           // pool capacity per query: K kept + room for new candidates
 
     const int lane = fgc_lane();
-    const int wv = threadIdx.x >> 6;
+    // wave index made explicitly uniform: everything derived from it (tile start, seed chunks, spans)
+    // then stays in scalar registers and scalar control flow
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int qbeg = (blockIdx.x * WPB + wv) * QT;
     if (qbeg >= a.n) return;  // no block-wide barrier is used below
     const int nq = min(QT, a.n - qbeg);
@@ -110,6 +112,14 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     if (a.sdir && isq) { unsigned char dd = a.sdir[qs]; qactive = !(dd == 0 || dd == 2); }
 
     unsigned long long nev = 0;
+#ifdef FGC_KNN_TIMERS
+    unsigned long long tm_cull = 0, tm_eval = 0, tm_pool = 0, tm_epi = 0, tm_total = clock64(), tm0;
+#define TM_START() tm0 = clock64()
+#define TM_STOP(acc) acc += clock64() - tm0
+#else
+#define TM_START()
+#define TM_STOP(acc)
+#endif
     unsigned nchunks = 0, nprunes = 0;
     const int slack = max(K >> 2, 4);   // a prune may keep up to K + slack candidates
 
@@ -329,6 +339,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                 const int c = cb + lane;
                 const bool cv = (c <= c1) && (c < sk0 || c > sk1);
                 unsigned mymask = cv ? (unsigned)act : 0u;   // queries (bit q) that need chunk c
+                TM_START();
                 if (cull) {
                     // per-chunk bounding-box test, lane = chunk
                     float blo[DR], bhi[DR];
@@ -355,6 +366,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                         if (cv && !(g2 > t)) mymask |= 1u << q;
                     }
                 }
+                TM_STOP(tm_cull);
                 for (unsigned long long any = fgc_ballot(mymask != 0u); any;) {
                     const int l = __ffsll((long long)any) - 1;
                     any &= any - 1;
@@ -374,6 +386,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     nev += (unsigned long long)__popcll(cact) * (unsigned)(min(j1, base + 64) - max(j0, base));
                     nchunks++;
                     for (unsigned long long m = cact; m;) {
+                        TM_START();
                         const int q = __ffsll((long long)m) - 1;
                         m &= m - 1;
                         const float t = fgc_readlane_f(tau, q);
@@ -395,7 +408,9 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                             }
                         }
                         unsigned long long pm = fgc_ballot(dsq < t);
+                        TM_STOP(tm_eval);
                         if (!pm) continue;
+                        TM_START();
                         // ---- append the passing lanes to query q's pool, pruning when it runs full: first to
                         //      a tighter threshold, then (if that is not enough) down to exactly K ----
                         int pc = fgc_readlane_i(cnt, q);
@@ -433,6 +448,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                         }
                         // keep tau tight: prune as soon as the pool is nearly full
                         if (pc > CAP - PRUNE_MARGIN || (pc > K && !(fgc_readlane_f(tau, q) < INFINITY))) prune(q, false);
+                        TM_STOP(tm_pool);
                     }
                 }
             }
@@ -441,7 +457,13 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 
     // ---- per query: cut the pool to exactly K, sort by distance, write the row at the query's
     //      original position (slot 0 = the query itself) ----
+    TM_START();
+#ifdef FGC_EXPERIMENT_NO_EPILOGUE
+    if (lane < nq) a.out_dist[(long long)a.order[qbeg + lane] * K] = tau;
+    for (int q = 0; q < 0; q++) {
+#else
     for (int q = 0; q < nq; q++) {
+#endif
         const int self = qbeg + q;
         const long long orig_q = (long long)a.order[self];
         prune(q, true);
@@ -511,7 +533,12 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             }
         }
     }
+    TM_STOP(tm_epi);
     if (a.stats && lane == 0) {
+#ifdef FGC_KNN_TIMERS
+        atomicAdd(&a.stats[3], tm_cull); atomicAdd(&a.stats[4], tm_eval); atomicAdd(&a.stats[5], tm_pool);
+        atomicAdd(&a.stats[6], tm_epi); atomicAdd(&a.stats[7], (unsigned long long)clock64() - tm_total);
+#endif
         atomicAdd(&a.stats[0], nev);
         atomicAdd(&a.stats[1], (unsigned long long)nchunks);
         atomicAdd(&a.stats[2], (unsigned long long)nprunes);

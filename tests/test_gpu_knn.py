@@ -148,3 +148,44 @@ def test_argument_errors():
         binned_select_knn(3, c, rs)
     with pytest.raises(RuntimeError):
         binned_select_knn(3, torch.rand(10, 3), torch.tensor([0, 10]))
+
+
+@pytest.mark.parametrize("n,K", [(1, 1), (1, 5), (2, 3), (63, 64), (64, 64), (65, 64), (129, 7)])
+def test_tiny_inputs(oracle, n, K):
+    rng = np.random.default_rng(n * 100 + K)
+    coords = rng.random((n, 3)).astype(np.float32)
+    gi, gd = _check(oracle, K, coords, [0, n])
+    check_knn_properties(gi, gd, coords, [0, n], K)
+
+
+def test_all_points_coincident(oracle):
+    coords = np.full((700, 3), 0.25, dtype=np.float32)
+    gi, gd = _gpu_knn(10, coords, [0, 300, 700])
+    check_knn_properties(gi, gd, coords, [0, 300, 700], 10)
+    assert (gd == 0).all()
+    oi, od = oracle.binned_select_knn(10, coords, [0, 300, 700])
+    np.testing.assert_array_equal(od, gd)
+
+
+def test_one_dense_cluster_plus_outliers(oracle):
+    # extreme imbalance: almost every point in one bin, a few far away (large dynamic range)
+    rng = np.random.default_rng(21)
+    coords = (rng.standard_normal((20000, 3)) * 1e-3).astype(np.float32)
+    coords[:5] = np.array([[50, 50, 50], [-40, 10, 0], [0, 0, 99], [7, -80, 3], [1, 1, 1]], np.float32)
+    gi, gd = _check(oracle, 32, coords, [0, 20000])
+    check_knn_properties(gi, gd, coords, [0, 20000], 32)
+
+
+def test_single_bin_per_dimension(oracle):
+    rng = np.random.default_rng(22)
+    coords = rng.random((3000, 4)).astype(np.float32)
+    _check(oracle, 9, coords, [0, 1000, 3000], n_bins=torch.tensor(1, device="cuda"))
+    _check(oracle, 9, coords, [0, 1000, 3000], n_bins=torch.tensor(2, device="cuda"))
+
+
+def test_many_events_with_one_point(oracle):
+    rng = np.random.default_rng(23)
+    coords = rng.random((200, 3)).astype(np.float32)
+    rs = np.arange(0, 201, dtype=np.int64)          # 200 events of one point each
+    gi, gd = _check(oracle, 4, coords, rs)
+    assert (gi[:, 0] == np.arange(200)).all() and (gi[:, 1:] == -1).all()
