@@ -1,0 +1,364 @@
+"""Dispatcher registration of the ops behind the Python wrappers.
+
+The reference registers its C++ kernels as torch ops and its wrappers call
+them through `torch.ops.*`, which is what makes the wrappers and GravNetOp
+TorchScript-scriptable (fastgraphcompute/extensions/bin_by_coordinates.cpp:
+143-153, index_replacer.cpp:43-53, binned_select_knn_grad.cpp:58-70,
+binned_knn_autograd_kernel.cpp:271-277).  The same schemas are registered here
+with `torch.library`; the implementations call libfgc_hip.so through ctypes.
+Two ops have no counterpart in the reference: the fused GravNet aggregation and
+the float32 select_with_default kernel.
+"""
+from typing import List, Optional, Tuple
+
+import torch
+
+from . import _lib, config
+
+_LIBS = []          # keep the Library objects alive
+last_stats = {}     # counters of the most recent kNN call when config.collect_stats is set
+
+
+def _define(ns: str, schema: str):
+    try:
+        lib = torch.library.Library(ns, "FRAGMENT")
+        lib.define(schema)
+    except RuntimeError as e:      # already defined (module imported twice under two names)
+        if "already" not in str(e) and "multiple" not in str(e).lower():
+            raise
+        lib = torch.library.Library(ns, "FRAGMENT")
+    _LIBS.append(lib)
+    return lib
+
+
+# ------------------------------------------------------------------ bin_by_coordinates
+def _bin_by_coordinates_impl(coordinates: torch.Tensor, row_splits: torch.Tensor, bin_width: Optional[torch.Tensor],
+                             n_bins: Optional[torch.Tensor], calc_n_per_bin: bool, pre_normalized: bool):
+    _lib.require_device(coordinates)
+    L = _lib.lib()
+    dev = coordinates.device
+    coords = coordinates.to(torch.float32).contiguous()
+    if coords.dim() != 2:
+        raise ValueError("coordinates must be [n_vert, n_coords]")
+    n, d = coords.shape
+    if d < 1 or d > 5:
+        raise ValueError("Unsupported number of binning dimensions.")
+    rs = row_splits.to(device=dev, dtype=torch.int64).contiguous()
+    n_rs = rs.numel()
+    if (bin_width is None or bin_width.numel() == 0) and (n_bins is None or n_bins.numel() == 0):
+        raise ValueError("Either bin_width or n_bins must be provided.")
+    nb_host = None
+    if n_bins is not None and n_bins.numel() > 0:
+        nb_t = n_bins.to(torch.int64).cpu()
+        if nb_t.dim() == 0:
+            nb_t = nb_t.repeat(d)
+        nb_host = [int(v) for v in nb_t.tolist()]
+        if len(nb_host) != d:
+            raise ValueError("bin_by_coordinates: coordinates.size(1) must be equal to nbins.size(0)")
+        if not all(v > 0 for v in nb_host):
+            raise ValueError("BinByCoordinates: n_bins must be greater than zero.")
+    bw_host = 0.0
+    have_bw = bin_width is not None and bin_width.numel() > 0
+    if have_bw:
+        if bin_width.numel() != 1:
+            raise ValueError("bin_by_coordinates: bin_width must be a singleton tensor")
+        bw_host = float(bin_width.to(torch.float32).reshape(-1)[0].item())
+        if not bw_host > 0:
+            raise ValueError("BinByCoordinates: bin_width must be greater than zero.")
+    if n == 0:
+        nb_out = torch.tensor(nb_host if nb_host is not None else [1] * d, dtype=torch.int64, device=dev)
+        B = int(torch.prod(nb_out).item()) * max(n_rs - 1, 0)
+        return (torch.empty((0, d + 1), dtype=torch.int64, device=dev),
+                torch.empty((0,), dtype=torch.int64, device=dev), nb_out,
+                torch.tensor([bw_host], dtype=torch.float32, device=dev),
+                torch.zeros((B,), dtype=torch.int64, device=dev))
+    geom = torch.empty(16, dtype=torch.float32, device=dev)
+    status = torch.zeros(4, dtype=torch.int32, device=dev)
+    ws_bytes = L.fgc_bin_geometry_workspace_bytes(n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    nb_arr = _lib.host_i64(nb_host if nb_host is not None else [1] * d)
+    with torch.cuda.device(dev):
+        st = _lib.stream_ptr()
+        _lib.check(L.fgc_bin_geometry_f32(_lib.ptr(coords), n, d, d, 1 if have_bw else 0, nb_arr,
+                                          1 if nb_host is not None else 0, bw_host, 1 if pre_normalized else 0,
+                                          _lib.ptr(geom), _lib.ptr(status), _lib.ptr(ws), ws_bytes, st))
+        g = geom.cpu()  # one synchronisation: n_bins sizes the outputs, the flags carry the input checks
+        flags = int(g[11:12].view(torch.int32).item())
+        if flags & _lib.ST_NONFINITE:
+            raise ValueError("BinByCoordinates: input coordinates contain non-finite values")
+        nb_final = [int(v) for v in g[6:6 + d].view(torch.int32).tolist()]
+        if flags & _lib.ST_BAD_RANGE:
+            if not all(v > 0 for v in nb_final):
+                raise ValueError("BinByCoordinates: n_bins must be greater than zero.")
+            raise ValueError("BinByCoordinates: dmax_coords must be greater than zero.")
+        B = max(n_rs - 1, 0)
+        for v in nb_final:
+            B *= v
+        assigned = torch.empty((n, d + 1), dtype=torch.int64, device=dev)
+        flat = torch.empty((n,), dtype=torch.int64, device=dev)
+        nper = torch.zeros((B,), dtype=torch.int64, device=dev)
+        _lib.check(L.fgc_bin_points_f32(_lib.ptr(coords), n, d, d, _lib.ptr(geom), _lib.ptr(rs), n_rs,
+                                        _lib.host_i64(nb_final), _lib.ptr(assigned), _lib.ptr(flat),
+                                        _lib.ptr(nper) if calc_n_per_bin else None, _lib.ptr(status), st))
+    nb_out = torch.tensor(nb_final, dtype=torch.int64, device=dev)
+    return assigned, flat, nb_out, geom[5:6].clone(), nper
+
+
+# ------------------------------------------------------------------ kNN forward / backward
+def calculate_optimal_bins(row_splits_host: torch.Tensor, K: int, max_bin_dims: int) -> int:
+    """n_bins heuristic of the reference (binned_knn_autograd_kernel.cpp:67-82),
+    evaluated with the same float32 tensor ops on the host: points per
+    row-split entry (the length of row_splits, not the number of events),
+    divided by K/32, to the power 1/dims, truncated, clamped to [5, 30]."""
+    rs = row_splits_host
+    if rs.numel() > 0:
+        elems = (torch.max(rs).to(torch.float32) / float(rs.numel()) + 1).to(torch.int64)
+    else:
+        elems = torch.tensor(1, dtype=torch.int64)
+    k32 = torch.tensor(float(K), dtype=torch.float32) / torch.tensor(32.0, dtype=torch.float32)
+    expo = torch.tensor(1.0, dtype=torch.float32) / torch.tensor(float(max_bin_dims), dtype=torch.float32)
+    n_bins = torch.pow(elems.to(torch.float32) / float(k32), float(expo)).to(torch.int64)
+    return int(torch.clamp(n_bins, 5, 30))
+
+
+def knn_grad(grad_distsq: torch.Tensor, idx: torch.Tensor, coords: torch.Tensor,
+             order: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _lib.require_device(grad_distsq, idx, coords)
+    L = _lib.lib()
+    g = grad_distsq.to(torch.float32).contiguous()
+    ii = idx.to(torch.int64).contiguous()
+    x = coords.to(torch.float32).contiguous()
+    n, D = x.shape
+    K = ii.shape[1]
+    out = torch.empty((n, D), dtype=torch.float32, device=x.device)
+    status = torch.zeros(4, dtype=torch.int32, device=x.device)
+    if order is not None:
+        order = order.to(device=x.device, dtype=torch.int32).contiguous()
+        if order.numel() != n:
+            raise ValueError("order must hold one entry per point")
+    with torch.cuda.device(x.device):
+        _lib.check(L.fgc_binned_select_knn_grad_f32(_lib.ptr(g), _lib.ptr(ii), _lib.ptr(x), _lib.ptr(out), n, K, D,
+                                                    _lib.ptr(order), _lib.ptr(status), _lib.stream_ptr()))
+    return out
+
+
+class _BinnedKNN(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, coords, row_splits, K, direction, n_bins, max_bin_dims, tf_compat):
+        _lib.require_device(coords)
+        if coords.dim() != 2 or coords.shape[1] == 0:
+            raise ValueError("Input coordinates must have at least one dimension.")
+        if max_bin_dims <= 0:
+            raise ValueError("max_bin_dims must be greater than 0.")
+        L = _lib.lib()
+        dev = coords.device
+        coords = coords.to(torch.float32).contiguous()
+        n, D = coords.shape
+        nbd = min(int(max_bin_dims), D)
+        if nbd < 2 or nbd > 5:
+            raise ValueError("Unsupported number of binning dimensions.")
+        if K < 1 or K > 256:
+            raise ValueError("binned_select_knn on MI355X supports 1 <= K <= 256, got %d" % K)
+        rs_host = row_splits.detach().to("cpu", torch.int64).contiguous()
+        n_rs = rs_host.numel()
+        if n_rs < 2:
+            raise ValueError("row_splits needs at least two entries")
+        if n_bins is None or n_bins.numel() == 0:
+            nb = [calculate_optimal_bins(rs_host, K, nbd)] * nbd
+        else:
+            nbt = n_bins.detach().to("cpu", torch.int64)
+            nb = [int(nbt.item())] * nbd if nbt.numel() == 1 else [int(v) for v in nbt.tolist()]
+            if len(nb) != nbd:
+                raise ValueError("bin_by_coordinates: coordinates.size(1) must be equal to nbins.size(0)")
+            if not all(v > 0 for v in nb):
+                raise RuntimeError("BinByCoordinates: n_bins must be greater than zero.")
+        rs_list = rs_host.tolist()
+        if n > 0 and (rs_list[0] != 0 or max(rs_list) != n or rs_list[-1] != n
+                      or any(b < a for a, b in zip(rs_list, rs_list[1:]))):
+            raise RuntimeError("Bin boundaries do not match row splits.")
+        rs_dev = row_splits if (row_splits.is_cuda and row_splits.dtype == torch.int64) else rs_host.to(dev)
+        rs_dev = rs_dev.contiguous()
+        idx = torch.empty((n, K), dtype=torch.int64, device=dev)
+        dist = torch.empty((n, K), dtype=torch.float32, device=dev)
+        order = torch.empty(0, dtype=torch.int32, device=dev)
+        if n > 0:
+            nb_arr = _lib.host_i64(nb)
+            rs_arr = _lib.host_i64(rs_list)
+            ws_bytes = L.fgc_binned_select_knn_workspace_bytes(n, D, nbd, nb_arr, n_rs, K)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            status = torch.zeros(4, dtype=torch.int32, device=dev)
+            stats = torch.zeros(8, dtype=torch.int64, device=dev) if config.collect_stats else None
+            dirt = None
+            if direction is not None and direction.numel() > 0:
+                dirt = direction.to(device=dev, dtype=torch.int64).contiguous()
+            with torch.cuda.device(dev):
+                st = _lib.stream_ptr()
+                _lib.check(L.fgc_binned_select_knn_f32(
+                    _lib.ptr(coords), n, D, _lib.ptr(rs_dev), rs_arr, n_rs, K, nbd, nb_arr, _lib.ptr(dirt),
+                    1 if tf_compat else 0, _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(status), _lib.ptr(stats),
+                    _lib.ptr(ws), ws_bytes, st))
+                if ctx.needs_input_grad[0]:
+                    # the backward processes queries in the forward's bin-sorted order
+                    order = torch.empty(n, dtype=torch.int32, device=dev)
+                    _lib.check(L.fgc_binned_knn_export_order_i32(n, D, rs_arr, n_rs, K, nbd, nb_arr,
+                                                                 1 if dirt is not None else 0, _lib.ptr(ws),
+                                                                 ws_bytes, _lib.ptr(order), st))
+            if config.sync_checks:
+                flags = int(status[0].item())
+                if flags & _lib.ST_NONFINITE:
+                    raise RuntimeError("BinByCoordinates: input coordinates contain non-finite values")
+                if flags & _lib.ST_BAD_RANGE:
+                    raise RuntimeError("BinByCoordinates: dmax_coords must be greater than zero.")
+            if stats is not None:
+                s = stats.tolist()
+                last_stats.update(distance_evaluations=s[0], candidate_chunks=s[1], pool_prunes=s[2],
+                                  n_bins=nb, n_vert=n, K=K, n_coords=D)
+        ctx.save_for_backward(idx, coords, order)
+        ctx.mark_non_differentiable(idx)
+        ctx.set_materialize_grads(False)   # no zero tensors for unused output gradients
+        return idx, dist
+
+    @staticmethod
+    def backward(ctx, _grad_idx, grad_dist):
+        idx, coords, order = ctx.saved_tensors
+        if not ctx.needs_input_grad[0]:
+            return None, None, None, None, None, None, None
+        if grad_dist is None:
+            return torch.zeros_like(coords), None, None, None, None, None, None
+        g = knn_grad(grad_dist, idx, coords, order if order.numel() else None)
+        return g, None, None, None, None, None, None
+
+
+def _knn_autograd_impl(coords, row_splits, K, direction, n_bins, max_bin_dims, torch_compatible_indices):
+    return _BinnedKNN.apply(coords, row_splits, K, direction, n_bins, max_bin_dims, torch_compatible_indices)
+
+
+def _knn_grad_impl(grad_distances, indices, distances, coordinates):
+    return knn_grad(grad_distances, indices, coordinates)
+
+
+# ------------------------------------------------------------------ index_replacer
+def _index_replacer_impl(to_be_replaced: torch.Tensor, replacements: torch.Tensor) -> torch.Tensor:
+    _lib.require_device(to_be_replaced, replacements)
+    L = _lib.lib()
+    src = to_be_replaced.contiguous()
+    rep = replacements.contiguous()
+    out = torch.empty_like(src)
+    with torch.cuda.device(src.device):
+        _lib.check(L.fgc_index_replacer_i64(_lib.ptr(src), _lib.ptr(rep), _lib.ptr(out), src.numel(), rep.numel(),
+                                            _lib.stream_ptr()))
+    return out
+
+
+# ------------------------------------------------------------------ select_with_default (float32 kernel)
+class _SelectWithDefault(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, idx, feat, default_value):
+        _lib.require_device(idx, feat)
+        L = _lib.lib()
+        ii = idx.to(torch.int64).contiguous()
+        ff = feat.contiguous()
+        V, K = ii.shape
+        rows, F = ff.shape
+        out = torch.empty((V, K, F), dtype=torch.float32, device=ff.device)
+        with torch.cuda.device(ff.device):
+            _lib.check(L.fgc_select_with_default_f32(_lib.ptr(ii), _lib.ptr(ff), _lib.ptr(out), V, K, F, rows,
+                                                     float(default_value), _lib.stream_ptr()))
+        ctx.save_for_backward(ii)
+        ctx.rows = rows
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        (ii,) = ctx.saved_tensors
+        if g is None or not ctx.needs_input_grad[1]:
+            return None, None, None
+        F = g.shape[-1]
+        valid = (ii != -1).reshape(-1)
+        tgt = torch.where(ii < 0, ii + ctx.rows, ii).reshape(-1)[valid]
+        gf = torch.zeros((ctx.rows, F), dtype=g.dtype, device=g.device)
+        gf.index_add_(0, tgt, g.reshape(-1, F)[valid])
+        return None, gf, None
+
+
+def _select_with_default_impl(idx, feat, default_value):
+    return _SelectWithDefault.apply(idx, feat, default_value)
+
+
+# ------------------------------------------------------------------ GravNet aggregation
+class _GravNetAggregate(torch.autograd.Function):
+    """(fmean, fmax) over the K neighbour slots of feat[idx] * exp(-10 distsq)."""
+
+    @staticmethod
+    def forward(ctx, idx, distsq, feat):
+        _lib.require_device(idx, distsq, feat)
+        L = _lib.lib()
+        ii = idx.to(torch.int64).contiguous()
+        d = distsq.to(torch.float32).contiguous()
+        f = feat.to(torch.float32).contiguous()
+        n, K = ii.shape
+        P = f.shape[1]
+        fmean = torch.empty((n, P), dtype=torch.float32, device=f.device)
+        fmax = torch.empty((n, P), dtype=torch.float32, device=f.device)
+        argmax = torch.empty((n, P), dtype=torch.int32, device=f.device)
+        with torch.cuda.device(f.device):
+            _lib.check(L.fgc_gravnet_aggregate_fwd_f32(_lib.ptr(ii), _lib.ptr(d), _lib.ptr(f), _lib.ptr(fmean),
+                                                       _lib.ptr(fmax), _lib.ptr(argmax), n, K, P, _lib.stream_ptr()))
+        ctx.save_for_backward(ii, d, f, argmax)
+        ctx.set_materialize_grads(False)
+        return fmean, fmax
+
+    @staticmethod
+    def backward(ctx, g_mean, g_max):
+        ii, d, f, argmax = ctx.saved_tensors
+        if g_mean is None and g_max is None:
+            return None, None, None
+        L = _lib.lib()
+        n, K = ii.shape
+        P = f.shape[1]
+        g_mean = torch.zeros((n, P), dtype=torch.float32, device=f.device) if g_mean is None \
+            else g_mean.to(torch.float32).contiguous()
+        g_max = torch.zeros((n, P), dtype=torch.float32, device=f.device) if g_max is None \
+            else g_max.to(torch.float32).contiguous()
+        g_feat = torch.zeros_like(f)
+        g_dist = torch.empty_like(d)
+        with torch.cuda.device(f.device):
+            _lib.check(L.fgc_gravnet_aggregate_bwd_f32(_lib.ptr(ii), _lib.ptr(d), _lib.ptr(f), _lib.ptr(argmax),
+                                                       _lib.ptr(g_mean), _lib.ptr(g_max), _lib.ptr(g_feat),
+                                                       _lib.ptr(g_dist), n, K, P, _lib.stream_ptr()))
+        return None, g_dist, g_feat
+
+
+def _gravnet_aggregate_impl(idx, distsq, feat):
+    return _GravNetAggregate.apply(idx, distsq, feat)
+
+
+# ------------------------------------------------------------------ registration
+def _register():
+    lib = _define("bin_by_coordinates",
+                  "bin_by_coordinates(Tensor coordinates, Tensor row_splits, Tensor? bin_width, Tensor? n_bins, "
+                  "bool calc_n_per_bin, bool pre_normalized) -> (Tensor, Tensor, Tensor, Tensor, Tensor)")
+    lib.impl("bin_by_coordinates", _bin_by_coordinates_impl, "CUDA")
+    lib.impl("bin_by_coordinates", _bin_by_coordinates_impl, "CPU")      # raises: no CPU fallback
+
+    lib = _define("index_replacer", "index_replacer(Tensor to_be_replaced, Tensor replacements) -> Tensor")
+    lib.impl("index_replacer", _index_replacer_impl, "CUDA")
+    lib.impl("index_replacer", _index_replacer_impl, "CPU")
+
+    lib = _define("binned_select_knn_grad",
+                  "binned_select_knn_grad(Tensor grad_distances, Tensor indices, Tensor distances, "
+                  "Tensor coordinates) -> Tensor")
+    lib.impl("binned_select_knn_grad", _knn_grad_impl, "CUDA")
+    lib.impl("binned_select_knn_grad", _knn_grad_impl, "CPU")
+
+    lib = _define("fastgraphcompute_custom_ops",
+                  "binned_select_knn_autograd(Tensor coords, Tensor row_splits, int K, Tensor? direction, "
+                  "Tensor? n_bins, int max_bin_dims, bool torch_compatible_indices) -> (Tensor, Tensor)")
+    lib.impl("binned_select_knn_autograd", _knn_autograd_impl, "Autograd")
+    lib.define("gravnet_aggregate(Tensor neighbor_idx, Tensor distsq, Tensor features) -> (Tensor, Tensor)")
+    lib.impl("gravnet_aggregate", _gravnet_aggregate_impl, "Autograd")
+    lib.define("select_with_default_f32(Tensor idx, Tensor feat, float default_value) -> Tensor")
+    lib.impl("select_with_default_f32", _select_with_default_impl, "Autograd")
+
+
+_register()

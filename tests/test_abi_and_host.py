@@ -55,13 +55,15 @@ def test_host_wrappers_reject_cpu_tensors_and_bad_arguments():
     import fastgraphcompute_amd as fgc
     with pytest.raises(RuntimeError):
         fgc.binned_select_knn(3, torch.rand(10, 3), torch.tensor([0, 10]))
-    with pytest.raises(ValueError):
+    # the wrapper is a scripted function like the reference's: its ValueErrors surface as torch.jit.Error,
+    # a RuntimeError
+    with pytest.raises((ValueError, RuntimeError, torch.jit.Error)):
         fgc.binned_select_knn(3, torch.rand(10, 0), torch.tensor([0, 10]))
-    with pytest.raises(ValueError):
+    with pytest.raises((ValueError, RuntimeError, torch.jit.Error)):
         fgc.binned_select_knn(3, torch.rand(10, 3), torch.tensor([0, 10]), max_bin_dims=0)
     with pytest.raises(RuntimeError):
         fgc.bin_by_coordinates(torch.rand(10, 3), torch.tensor([0, 10]), n_bins=4)
-    with pytest.raises(AssertionError):
+    with pytest.raises((AssertionError, RuntimeError, torch.jit.Error)):
         fgc.index_replacer(torch.zeros(3, dtype=torch.int32), torch.zeros(3, dtype=torch.int64))
     with pytest.raises(NotImplementedError):
         fgc.oc_helper_matrices()
@@ -95,3 +97,19 @@ def test_gravnet_module_state_dict_names():
         "space_transformations.weight", "space_transformations.bias", "propagate_transformations.weight",
         "propagate_transformations.bias", "output_transformations.0.weight", "output_transformations.0.bias"}
     assert op.output_transformations[0].in_features == 8 + 2 * 5
+
+
+def test_ops_are_registered_and_wrappers_script():
+    import fastgraphcompute_amd  # noqa: F401
+    from fastgraphcompute_amd.gnn_ops import GravNetOp
+    # the reference's dispatcher surface (same namespaces, names and schemas)
+    s = str(torch.ops.fastgraphcompute_custom_ops.binned_select_knn_autograd.default._schema)
+    assert "Tensor coords, Tensor row_splits, int K, Tensor? direction, Tensor? n_bins, int max_bin_dims, " \
+           "bool torch_compatible_indices" in s
+    assert "Tensor? bin_width, Tensor? n_bins, bool calc_n_per_bin, bool pre_normalized" in \
+        str(torch.ops.bin_by_coordinates.bin_by_coordinates.default._schema)
+    assert torch.ops.index_replacer.index_replacer is not None
+    assert torch.ops.binned_select_knn_grad.binned_select_knn_grad is not None
+    # scripting compiles without a device
+    sm = torch.jit.script(GravNetOp(8, 6, 3, 5, 4))
+    assert "binned_select_knn_autograd" in str(sm.graph) or "binned_select_knn" in str(sm.code)

