@@ -47,6 +47,17 @@ __device__ __forceinline__ int fgc_mbcnt(unsigned long long m)
                                           __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
 }
 
+// sum of v over the 64 lanes (returned in every lane): four DPP steps inside each row of 16 lanes
+// (quad swaps, half-row mirror, row mirror), then the four row sums are combined through scalar reads
+__device__ __forceinline__ float fgc_wave_sum(float v)
+{
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));   // quad_perm [1,0,3,2]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true));  // row_half_mirror
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true));  // row_mirror
+    return (fgc_readlane_f(v, 0) + fgc_readlane_f(v, 16)) + (fgc_readlane_f(v, 32) + fgc_readlane_f(v, 48));
+}
+
 // internal launchers shared between translation units (all enqueue on `s`)
 int fgc_fill_u32(void *d, uint32_t v, int64_t n_words, hipStream_t s);
 int fgc_copy_u32(void *dst, const void *src, int64_t n_words, hipStream_t s);

@@ -31,17 +31,25 @@ extern "C" int fgc_index_replacer_i64(const int64_t *d_in, const int64_t *d_repl
 // gradient of distsq wrt the coordinates
 // ---------------------------------------------------------------------------
 // g[m] += 2 gd[i,k] (x_m - x_i) for every neighbour m = idx[i,k] and
-// g[i] -= sum_k of the same terms.  A block takes GQ queries - consecutive in
-// the bin-sorted order when `order` is given, so their neighbourhoods overlap -
-// and first combines all contributions to the same target point in an LDS hash
-// table (open addressing, LDS float atomics); only the distinct targets go to
-// global memory, one float atomic per coordinate.  Pairs that find no slot
-// within a few probes go to global memory directly.
-#ifndef GQ
-#define GQ 64          // queries per block (4 wavefronts x GQ/4)
+// g[i] -= sum_k of the same terms.  A wavefront takes GW queries - consecutive
+// in the bin-sorted order when `order` is given, so their neighbourhoods
+// overlap - lane k owning neighbour slot k, and first combines all contributions
+// to the same target point in its own LDS hash table (open addressing).  The
+// neighbours of one query are distinct points, so the lanes of one instruction
+// never update the same table entry and, the table being private to the
+// wavefront, the update is a plain LDS read-add-write of one float4 - no float
+// atomics on chip.  Only the distinct targets of the wavefront go to global
+// memory, one float atomic per coordinate with a target's coordinates in
+// adjacent lanes.  Pairs that find no table slot within a few probes go to
+// global memory directly.
+#ifndef GW
+#define GW 16          // queries per wavefront
+#endif
+#ifndef GU
+#define GU 4           // queries a wavefront processes together (loads in flight)
 #endif
 #ifndef GRAD_H
-#define GRAD_H 2048     // hash table slots per block (upper bound, shrunk for wide points)
+#define GRAD_H 512     // hash table slots per wavefront (upper bound, shrunk for wide points)
 #endif
 #define GRAD_PROBES 8
 #define GRAD_EMPTY 0xffffffffu
@@ -51,18 +59,19 @@ __global__ __launch_bounds__(256) void k_knn_grad(const float *__restrict__ gd, 
                                                   const uint32_t *__restrict__ order, int64_t n, int K, int D,
                                                   int H, int *__restrict__ status)
 {
-    extern __shared__ unsigned char s_raw[];
-    unsigned *keys = (unsigned *)s_raw;            // [H]
-    float *vals = (float *)(s_raw + (size_t)H * 4);  // [H][D]
-    for (int t = threadIdx.x; t < H; t += 256) keys[t] = GRAD_EMPTY;
-    for (int t = threadIdx.x; t < H * D; t += 256) vals[t] = 0.f;
-    __syncthreads();
-
-    const int lane = fgc_lane(), wv = threadIdx.x >> 6;
+    extern __shared__ __align__(16) unsigned char s_raw[];
+    const int lane = fgc_lane();
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // uniform by construction
+    const int D4 = (D + 3) >> 2;                       // float4 groups per point
+    const size_t wave_bytes = (size_t)H * (4 + 16 * (size_t)D4);
+    float4 *vals = (float4 *)(s_raw + wave_bytes * wv);                  // [H][D4]
+    unsigned *keys = (unsigned *)(s_raw + wave_bytes * wv + (size_t)H * 16 * D4);   // [H]
+    for (int t = lane; t < H; t += 64) keys[t] = GRAD_EMPTY;
+    for (int t = lane; t < H * D4; t += 64) vals[t] = make_float4(0.f, 0.f, 0.f, 0.f);
     const unsigned hmask = (unsigned)H - 1u;
     bool bad = false;
 
-    // add v[0..D) to target m: LDS table if a slot is found, global memory otherwise
+    // slot of target m in the wavefront's table, or -1 when no slot is free within a few probes
     auto slot_of = [&](unsigned m) -> int {
         unsigned h = (m * 2654435761u) >> 7;
         for (int p = 0; p < GRAD_PROBES; p++) {
@@ -73,48 +82,83 @@ __global__ __launch_bounds__(256) void k_knn_grad(const float *__restrict__ gd, 
         return -1;
     };
 
-    for (int qq = wv; qq < GQ; qq += 4) {
-        const int64_t pos = (int64_t)blockIdx.x * GQ + qq;
-        if (pos >= n) break;   // wave-uniform
-        const int64_t i = order ? (int64_t)order[pos] : pos;
-        // the query's own slot (its contribution is the negated sum over its row)
-        int self_slot = 0;
-        if (lane == 0) self_slot = slot_of((unsigned)i);
-        self_slot = fgc_readlane_i(self_slot, 0);
+    const int64_t wave0 = ((int64_t)blockIdx.x * 4 + wv) * GW;
+    for (int q0 = 0; q0 < GW; q0 += GU) {
+        int64_t qi[GU];
+        bool qv[GU];
+#pragma unroll
+        for (int u = 0; u < GU; u++) {
+            const int64_t pos = wave0 + q0 + u;
+            qv[u] = pos < n;
+            qi[u] = qv[u] ? (order ? (int64_t)order[pos] : pos) : 0;
+        }
         for (int k0 = 0; k0 < K; k0 += 64) {
             const int k = k0 + lane;
-            int64_t m = -1;
-            float g = 0.f;
-            if (k < K) { m = idx[i * K + k]; g = gd[i * K + k]; }
-            if (m >= n) { bad = true; m = -1; }
-            const bool on = m >= 0;
-            const int sl = on ? slot_of((unsigned)m) : -1;
-            for (int c = 0; c < D; c++) {
-                const float xi = x[i * D + c];
-                float add = 0.f;
-                if (on) {
-                    add = 2.f * g * (x[m * D + c] - xi);
-                    if (sl >= 0) atomicAdd(&vals[sl * D + c], add);
-                    else atomicAdd(&gx[m * D + c], add);
-                }
-                float self = add;
+            int64_t m[GU];
+            float g[GU];
+            int sl[GU];
 #pragma unroll
-                for (int o = 32; o > 0; o >>= 1) self += __shfl_xor(self, o, 64);
-                if (lane == 0) {
-                    if (self_slot >= 0) atomicAdd(&vals[self_slot * D + c], -self);
-                    else atomicAdd(&gx[i * D + c], -self);
+            for (int u = 0; u < GU; u++) {
+                m[u] = -1; g[u] = 0.f;
+                if (k < K && qv[u]) { m[u] = idx[qi[u] * K + k]; g[u] = gd[qi[u] * K + k]; }
+            }
+#pragma unroll
+            for (int u = 0; u < GU; u++) {
+                if (m[u] >= n) { bad = true; m[u] = -1; }
+                sl[u] = (m[u] >= 0) ? slot_of((unsigned)m[u]) : -1;
+            }
+            for (int c4 = 0; c4 < D4; c4++) {
+#pragma unroll
+                for (int u = 0; u < GU; u++) {
+                    float add[4], self[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int c = c4 * 4 + e;
+                        add[e] = 0.f;
+                        if (c < D && m[u] >= 0) add[e] = 2.f * g[u] * (x[m[u] * D + c] - x[qi[u] * D + c]);
+                        self[e] = (c < D) ? fgc_wave_sum(add[e]) : 0.f;
+                    }
+                    if (m[u] >= 0) {
+                        if (sl[u] >= 0) {
+                            // distinct targets within the instruction, private table: plain read-add-write
+                            float4 v = vals[sl[u] * D4 + c4];
+                            v.x += add[0]; v.y += add[1]; v.z += add[2]; v.w += add[3];
+                            vals[sl[u] * D4 + c4] = v;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (c4 * 4 + e < D) atomicAdd(&gx[m[u] * D + c4 * 4 + e], add[e]);
+                        }
+                    }
+                    // the query's own share, after the neighbours' updates of this instruction
+                    if (qv[u]) {
+                        int ss = -1;
+                        if (lane == 0) ss = slot_of((unsigned)qi[u]);
+                        ss = fgc_readlane_i(ss, 0);
+                        if (lane == 0) {
+                            if (ss >= 0) {
+                                float4 v = vals[ss * D4 + c4];
+                                v.x -= self[0]; v.y -= self[1]; v.z -= self[2]; v.w -= self[3];
+                                vals[ss * D4 + c4] = v;
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 4; e++)
+                                    if (c4 * 4 + e < D) atomicAdd(&gx[qi[u] * D + c4 * 4 + e], -self[e]);
+                            }
+                        }
+                    }
                 }
             }
         }
     }
-    __syncthreads();
-    // one lane per (slot, coordinate): the atomics of one target sit in adjacent lanes
-    for (int t = threadIdx.x; t < H * D; t += 256) {
-        const int sl = t / D;
+    // flush: one lane per (slot, coordinate), the atomics of one target sit in adjacent lanes
+    const float *vflat = (const float *)vals;
+    for (int t = lane; t < H * D4 * 4; t += 64) {
+        const int sl = t / (D4 * 4), c = t - sl * (D4 * 4);
         const unsigned m = keys[sl];
-        if (m == GRAD_EMPTY) continue;
-        const float v = vals[t];
-        if (v != 0.f) atomicAdd(&gx[(int64_t)m * D + (t - sl * D)], v);
+        if (m == GRAD_EMPTY || c >= D) continue;
+        const float v = vflat[t];
+        if (v != 0.f) atomicAdd(&gx[(int64_t)m * D + c], v);
     }
     if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
 }
@@ -122,7 +166,8 @@ __global__ __launch_bounds__(256) void k_knn_grad(const float *__restrict__ gd, 
 static int grad_table_size(int D)
 {
     int H = GRAD_H;
-    while (H > 64 && (size_t)H * (4 + 4 * (size_t)D) > 65536) H >>= 1;
+    const size_t d4 = (size_t)((D + 3) / 4);
+    while (H > 64 && 4 * (size_t)H * (4 + 16 * d4) > 49152) H >>= 1;
     return H;
 }
 
@@ -131,15 +176,15 @@ extern "C" int fgc_binned_select_knn_grad_f32(const float *d_grad_distsq, const 
                                               int32_t K, int32_t n_coords, const int32_t *d_order,
                                               int32_t *d_status, void *stream)
 {
-    if (n_vert < 0 || K < 1 || n_coords < 1 || n_coords > 2048) return FGC_EINVAL;
+    if (n_vert < 0 || K < 1 || n_coords < 1 || n_coords > 128) return FGC_EINVAL;
     if (n_vert >= (1ll << 32) - 1) return FGC_EINVAL;
     if (n_vert == 0) return FGC_OK;
     hipStream_t s = (hipStream_t)stream;
     int rc = fgc_fill_u32(d_grad_coords, 0u, n_vert * n_coords, s);
     if (rc) return rc;
     const int H = grad_table_size(n_coords);
-    const size_t lds = (size_t)H * (4 + 4 * (size_t)n_coords);
-    const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GQ);
+    const size_t lds = 4 * (size_t)H * (4 + 16 * (size_t)((n_coords + 3) / 4));
+    const unsigned blocks = (unsigned)fgc_cdiv(n_vert, 4 * GW);
     hipLaunchKernelGGL(k_knn_grad, dim3(blocks), dim3(256), lds, s, d_grad_distsq, d_idx, d_coords,
                        d_grad_coords, (const uint32_t *)d_order, n_vert, (int)K, (int)n_coords, H, d_status);
     FGC_LAUNCH_CHECK();
