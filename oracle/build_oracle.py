@@ -19,6 +19,8 @@ REF_TUS = [
     "binned_select_knn_cpu.cpp",
     "binned_select_knn_grad_cpu.cpp",
     "index_replacer_cpu.cpp",
+    "oc_helper_cpu.cpp",
+    "oc_helper_helper.cpp",
 ]
 
 
@@ -33,7 +35,7 @@ def build_oracle(verbose=True):
 
 
 def build_ref(ref_root, verbose=True):
-    """Compile the reference's four CPU kernel translation units (they need
+    """Compile the reference's CPU kernel translation units (they need
     only the installed libtorch headers) and link them with ref_driver.cpp."""
     src_dir = os.path.join(ref_root, "fastgraphcompute", "extensions")
     if not os.path.isdir(src_dir):

@@ -360,6 +360,45 @@ void fgc_oracle_knn_brute(const float *coord, const int64_t *row_splits,
     }
 }
 
+/* Object/vertex index matrices of the object-condensation helper
+ * (calc_m, oc_helper_cpu.cpp:17-82).  For object k = (unique_idx[k], row split
+ * unique_rs_asso[k]): M[k, :] lists, in ascending order, the vertices of that
+ * row split whose association index equals unique_idx[k]; M_not[k, :] those
+ * whose index differs; both padded with -1.  The reference fills transposed
+ * buffers and transposes afterwards (oc_helper_cpu.cpp:150-151); the result is
+ * the row-major [n_unique, n_max*] layout written here directly.  A row that
+ * would overflow its width is cut at the width (the reference warns and stops
+ * one element later, outside the buffer).  Returns the number of cut rows. */
+int64_t fgc_oracle_oc_calc_m(const int64_t *asso_idx, const int64_t *unique_idx,
+                             const int64_t *unique_rs_asso, const int64_t *rs,
+                             int64_t *M, int64_t *M_not, int64_t n_vert, int64_t n_unique,
+                             int64_t n_maxuq, int64_t n_maxrs, int calc_m_not)
+{
+    int64_t cut = 0;
+    for (int64_t k = 0; k < n_unique; k++) {
+        int64_t uq = unique_idx[k];
+        int64_t r = unique_rs_asso[k];
+        int64_t lo = rs[r], hi = rs[r + 1];
+        if (hi > n_vert) hi = n_vert;
+        int64_t fill = 0;
+        for (int64_t v = lo; v < hi; v++)
+            if (asso_idx[v] == uq) {
+                if (fill >= n_maxuq) { cut++; break; }
+                M[k * n_maxuq + fill++] = v;
+            }
+        for (; fill < n_maxuq; fill++) M[k * n_maxuq + fill] = -1;
+        if (!calc_m_not) continue;
+        fill = 0;
+        for (int64_t v = lo; v < hi; v++)
+            if (asso_idx[v] != uq) {
+                if (fill >= n_maxrs) { cut++; break; }
+                M_not[k * n_maxrs + fill++] = v;
+            }
+        for (; fill < n_maxrs; fill++) M_not[k * n_maxrs + fill] = -1;
+    }
+    return cut;
+}
+
 int fgc_oracle_max_threads(void)
 {
 #ifdef _OPENMP

@@ -36,6 +36,19 @@ Pinning status (what fixes each function independently of this restatement):
                                    shapes and script-vs-eager only), so the C
                                    aggregation kernel is pinned against that
                                    torch composition and autograd.
+  oc_helper_inputs,
+  max_same_valued_entries_per_row_split
+                                   numpy.unique per row split, the routine the
+                                   reference's own test restates them with
+                                   (tests/test_oc_helper_helper.py:63-111); the
+                                   known answers of tests/test_oc_helper.py:
+                                   55-57 and the reference's compiled
+                                   oc_helper_helper.cpp (oracle/_ref).
+  oc_calc_m / oc_helper_matrices   the hand-written expectation of tests/
+                                   test_oc_helper.py:80-112, the stored
+                                   matrices tests/test_oc_helper_large_M*.npy
+                                   (:205-230), the reference's compiled calc_m
+                                   (oracle/_ref) element for element.
 """
 import ctypes
 import os
@@ -399,3 +412,107 @@ def gravnet_forward_torch(x, row_splits, weights, k, n_threads=8):
     out = torch.relu(lin(cat, weights["output_transformations.0.weight"],
                          weights["output_transformations.0.bias"]))
     return out, idx, distsq, space
+
+
+# --------------------------------------------------------------------------
+# object-condensation helper matrices
+# --------------------------------------------------------------------------
+def max_same_valued_entries_per_row_split(asso_idx, row_splits, filter_negative=True, use_ref=False):
+    """oc_helper_helper.cpp:30-94: per row split the largest multiplicity of one value and the number of
+    distinct values (negative values dropped first when filter_negative), and the maximum over the splits."""
+    a = _c(asso_idx, np.int64)
+    rs = _c(row_splits, np.int64)
+    n_rs = len(rs) - 1
+    mx = np.zeros(n_rs, dtype=np.int64)
+    nobj = np.zeros(n_rs, dtype=np.int64)
+    if use_ref:
+        g = np.zeros(1, dtype=np.int64)
+        rc = ref_lib().fgc_ref_max_same_valued(_ip(a), _ip(rs), _ip(mx), _ip(g), _ip(nobj),
+                                               ctypes.c_int64(a.size), ctypes.c_int64(len(rs)),
+                                               ctypes.c_int(int(filter_negative)))
+        if rc:
+            raise RuntimeError("reference max_same_valued_entries_per_row_split raised")
+        return mx, int(g[0]), nobj
+    for r in range(n_rs):
+        sl = a[rs[r]:rs[r + 1]]
+        if filter_negative:
+            sl = sl[sl >= 0]
+        if sl.size == 0:
+            continue
+        vals, counts = np.unique(sl, return_counts=True)
+        mx[r] = counts.max()
+        nobj[r] = vals.size
+    return mx, int(mx.max()) if n_rs > 0 else 0, nobj
+
+
+def oc_helper_inputs(truth_indices, row_splits, filter_negative=True):
+    """_helper_inputs, oc_helper.py:18-149: the distinct (value, row split) pairs with value != -1 (and >= 0
+    when filter_negative), here ordered by (row split, value); the reference orders them by an unstable argsort
+    over the row split (oc_helper.py:196-198), so only the set of pairs is defined.  Returns (unique_vals,
+    unique_row_splits, max_same_unique_per_split, lengths, max_length, objects_per_split)."""
+    a = _c(truth_indices, np.int64)
+    rs = _c(row_splits, np.int64)
+    lengths = rs[1:] - rs[:-1]
+    uv, ur = [], []
+    for r in range(len(rs) - 1):
+        sl = a[rs[r]:rs[r + 1]]
+        sl = sl[sl != -1]
+        if filter_negative:
+            sl = sl[sl >= 0]
+        v = np.unique(sl)
+        uv.append(v)
+        ur.append(np.full(v.size, r, dtype=np.int64))
+    uv = np.concatenate(uv) if uv else np.zeros(0, np.int64)
+    ur = np.concatenate(ur) if ur else np.zeros(0, np.int64)
+    _, gmax, nobj = max_same_valued_entries_per_row_split(a, rs, filter_negative)
+    return uv, ur, gmax, lengths, int(lengths.max()), nobj
+
+
+def oc_calc_m(asso_idx, unique_idx, unique_rs_asso, row_splits, n_maxuq, n_maxrs, calc_m_not=True,
+              use_ref=False):
+    """oc_helper_cpu, oc_helper_cpu.cpp:118-156 (calc_m :17-82).  Returns (M [U, n_maxuq], M_not [U, n_maxrs]
+    or None when calc_m_not is False: the reference leaves that buffer uninitialised on the CPU and returns a
+    [0, 0] tensor from its CUDA twin, oc_helper_cuda_kernel.cu:171-176)."""
+    a = _c(asso_idx, np.int64)
+    uq = _c(unique_idx, np.int64)
+    ur = _c(unique_rs_asso, np.int64)
+    rs = _c(row_splits, np.int64)
+    U = uq.size
+    M = np.empty((U, n_maxuq), dtype=np.int64)
+    M_not = np.empty((U, n_maxrs), dtype=np.int64) if calc_m_not else None
+    if use_ref:
+        rc = ref_lib().fgc_ref_oc_helper(_ip(a), _ip(uq), _ip(ur), _ip(rs), _ip(M), _ip(M_not),
+                                         ctypes.c_int64(a.size), ctypes.c_int64(U), ctypes.c_int64(len(rs)),
+                                         ctypes.c_int64(n_maxuq), ctypes.c_int64(n_maxrs),
+                                         ctypes.c_int(int(calc_m_not)))
+        if rc:
+            raise RuntimeError("reference oc_helper_cpu raised")
+        return M, M_not
+    f = lib().fgc_oracle_oc_calc_m
+    f.restype = ctypes.c_int64
+    f(_ip(a), _ip(uq), _ip(ur), _ip(rs), _ip(M), _ip(M_not), ctypes.c_int64(a.size), ctypes.c_int64(U),
+      ctypes.c_int64(n_maxuq), ctypes.c_int64(n_maxrs), ctypes.c_int(int(calc_m_not)))
+    return M, M_not
+
+
+def oc_helper_matrices(truth_idxs, row_splits, calc_m_not=True, use_ref=False):
+    """oc_helper_matrices, oc_helper.py:152-229: (M, M_not, objects_per_split); rows ordered by (row split,
+    value)."""
+    uv, ur, gmax, _lengths, max_len, nobj = oc_helper_inputs(truth_idxs, row_splits, True)
+    M, M_not = oc_calc_m(truth_idxs, uv, ur, row_splits, gmax, max_len, calc_m_not, use_ref=use_ref)
+    return M, M_not, nobj
+
+
+def oc_sort_rows(M, M_not):
+    """The canonical form the reference's tests compare in (tests/test_oc_helper.py:11-26): entries of every
+    row ascending with -1 last, rows ordered by their first M entry."""
+    def rows_sorted(A):
+        if A.size == 0:
+            return A
+        big = A.max() + 100
+        key = np.where(A == -1, big, A)
+        return np.take_along_axis(A, np.argsort(key, axis=1, kind="stable"), axis=1)
+    M = rows_sorted(np.asarray(M))
+    M_not = rows_sorted(np.asarray(M_not)) if M_not is not None else None
+    order = np.argsort(M[:, 0], kind="stable") if M.size else np.arange(M.shape[0])
+    return M[order], (M_not[order] if M_not is not None else None)

@@ -1,8 +1,9 @@
 // C-ABI driver around the reference's own CPU kernels (test infrastructure).
 //
-// The four functions declared below are defined by the reference's sources
+// The functions declared below are defined by the reference's sources
 // (bin_by_coordinates_cpu.cpp:102, binned_select_knn_cpu.cpp:211,
-// binned_select_knn_grad_cpu.cpp:96, index_replacer_cpu.cpp:28), which
+// binned_select_knn_grad_cpu.cpp:96, index_replacer_cpu.cpp:28,
+// oc_helper_cpu.cpp:118, oc_helper_helper.cpp:30), which
 // oracle/build_oracle.py compiles unmodified from the reference checkout.
 // This file only wraps caller memory in tensors and copies results out, so
 // that the checker can call them through ctypes without registering torch
@@ -28,6 +29,14 @@ torch::Tensor binned_select_knn_grad_cpu_fn(torch::Tensor grad_distances,
 
 torch::Tensor index_replacer_cpu_fn(torch::Tensor to_be_replaced,
                                     torch::Tensor replacements);
+
+// oc_helper_cpu.cpp:118 and oc_helper_helper.cpp:30
+std::tuple<torch::Tensor, torch::Tensor> oc_helper_cpu(
+    torch::Tensor asso_idx, torch::Tensor unique_idx, torch::Tensor unique_rs_asso, torch::Tensor rs,
+    torch::Tensor max_n_unique_over_splits, torch::Tensor max_n_in_splits, bool calc_m_not);
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> max_same_valued_entries_per_row_split(
+    const torch::Tensor &asso_idx, torch::Tensor row_splits, bool filter_negative);
 
 namespace {
 torch::Tensor f32(const float *p, std::initializer_list<int64_t> s) {
@@ -94,6 +103,36 @@ int fgc_ref_index_replacer(const int64_t *in, const int64_t *repl, int64_t *out,
     try {
         auto r = index_replacer_cpu_fn(i64(in, {n}), i64(repl, {n_repl}));
         copy_out<int64_t>(r, out);
+        return 0;
+    } catch (...) { return 1; }
+}
+
+// M [n_unique, n_maxuq] and M_not [n_unique, n_maxrs] of oc_helper_cpu (M_not is left untouched when
+// calc_m_not is 0: the reference returns uninitialised memory for it then)
+int fgc_ref_oc_helper(const int64_t *asso, const int64_t *unique_idx, const int64_t *unique_rs,
+                      const int64_t *rs, int64_t *M, int64_t *M_not, int64_t n_vert, int64_t n_unique,
+                      int64_t n_rs, int64_t n_maxuq, int64_t n_maxrs, int calc_m_not) {
+    try {
+        auto uq = torch::full({1}, n_maxuq, torch::kInt64);
+        auto mrs = torch::full({1}, n_maxrs, torch::kInt64);
+        auto r = oc_helper_cpu(i64(asso, {n_vert}), i64(unique_idx, {n_unique}), i64(unique_rs, {n_unique}),
+                               i64(rs, {n_rs}), uq, mrs, calc_m_not != 0);
+        copy_out<int64_t>(std::get<0>(r), M);
+        if (calc_m_not) copy_out<int64_t>(std::get<1>(r), M_not);
+        return 0;
+    } catch (...) { return 1; }
+}
+
+// max_per_split [n_rs-1], global_max [1], objects_per_split [n_rs-1]
+int fgc_ref_max_same_valued(const int64_t *asso, const int64_t *rs, int64_t *max_per_split,
+                            int64_t *global_max, int64_t *objects_per_split, int64_t n_vert, int64_t n_rs,
+                            int filter_negative) {
+    try {
+        auto r = max_same_valued_entries_per_row_split(i64(asso, {n_vert}), i64(rs, {n_rs}),
+                                                       filter_negative != 0);
+        copy_out<int64_t>(std::get<0>(r), max_per_split);
+        global_max[0] = std::get<1>(r).item<int64_t>();
+        copy_out<int64_t>(std::get<2>(r), objects_per_split);
         return 0;
     } catch (...) { return 1; }
 }

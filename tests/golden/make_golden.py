@@ -1,6 +1,6 @@
-"""Writes tests/golden/ref_cpu_kernels.npz: outputs of the reference's own CPU
-kernels (compiled from the reference checkout into oracle/_ref by
-oracle/build_oracle.py) on small seeded inputs.  Run in the build container,
+"""Writes tests/golden/ref_cpu_kernels.npz and tests/golden/ref_oc_helper.npz:
+outputs of the reference's own CPU kernels (compiled from the reference
+checkout into oracle/_ref by oracle/build_oracle.py) on small seeded inputs.  Run in the build container,
 where the reference checkout exists:
 
     python oracle/build_oracle.py && python tests/golden/make_golden.py
@@ -44,6 +44,48 @@ def make_inputs(name, n, D, K, rsf, dist):
     return c, rs
 
 
+def oc_cases():
+    """name -> (association indices, row splits) of the object-condensation helper cases."""
+    import torch
+    cases = {}
+    cases["hand"] = (np.array([3, 7, 3, -1, -1, 3, 7, 1, 1, 0, 0, -1, 1, 1, -1, 3, -1, 19, 3, 2, -1, 19]),
+                     np.array([0, 15, 22]))               # tests/test_oc_helper.py:31-37
+    torch.manual_seed(42)                                 # tests/test_oc_helper.py:201-210
+    a = (torch.randint(0, 100, (1000,), dtype=torch.int64, device="cpu") - 1).numpy()
+    cases["stored"] = (a, np.array([0, 250, 500, 1000]))
+    rng = np.random.default_rng(4242)
+    a = rng.integers(-3, 400, 6000)
+    cases["ragged"] = (a, np.array([0, 1, 1, 700, 2500, 2501, 6000]))
+    a = rng.integers(0, 60, 3000) * 1234567890123 + 5     # values that need more than 32 bits
+    a[rng.random(3000) < 0.2] = -1
+    cases["wide_values"] = (a, np.array([0, 1000, 3000]))
+    cases["all_negative"] = (np.full(50, -1), np.array([0, 20, 50]))
+    cases["single"] = (np.array([7]), np.array([0, 1]))
+    cases["one_object"] = (np.full(300, 5), np.array([0, 300]))
+    return {k: (np.asarray(v[0], np.int64), np.asarray(v[1], np.int64)) for k, v in cases.items()}
+
+
+def make_oc():
+    out = {}
+    for name, (a, rs) in oc_cases().items():
+        uv, ur, gmax, lengths, max_len, nobj = O.oc_helper_inputs(a, rs, True)
+        M, M_not = O.oc_calc_m(a, uv, ur, rs, gmax, max_len, True, use_ref=True)
+        out[name + "/asso"] = a
+        out[name + "/row_splits"] = rs
+        out[name + "/unique_idx"] = uv
+        out[name + "/unique_rs"] = ur
+        out[name + "/M"] = M
+        out[name + "/M_not"] = M_not.astype(np.int32)
+        for flt in (True, False):
+            mx, g, no = O.max_same_valued_entries_per_row_split(a, rs, flt, use_ref=True)
+            tag = "/filter" if flt else "/nofilter"
+            out[name + tag + "_max_per_split"] = mx
+            out[name + tag + "_global_max"] = np.int64(g)
+            out[name + tag + "_objects_per_split"] = no
+    np.savez_compressed(os.path.join(HERE, "ref_oc_helper.npz"), **out)
+    print("wrote", os.path.join(HERE, "ref_oc_helper.npz"))
+
+
 def main():
     if O.ref_lib() is None:
         raise SystemExit("oracle/_ref/libfgc_ref.so missing: run python oracle/build_oracle.py first")
@@ -74,6 +116,7 @@ def main():
         out[name + "/grad_coords"] = g
     np.savez_compressed(os.path.join(HERE, "ref_cpu_kernels.npz"), **out)
     print("wrote", os.path.join(HERE, "ref_cpu_kernels.npz"))
+    make_oc()
 
 
 if __name__ == "__main__":
