@@ -38,9 +38,14 @@ SIGNATURES = {
     "fgc_gravnet_aggregate_fwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp]),
     "fgc_gravnet_aggregate_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32,
                                                      _vp]),
+    "fgc_oc_helper_workspace_bytes": (ctypes.c_size_t, [_i64]),
+    "fgc_oc_helper_objects_i64": (ctypes.c_int, [_vp, _i64, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp,
+                                                 ctypes.c_size_t, _vp]),
+    "fgc_oc_helper_fill_i64": (ctypes.c_int, [_i64, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                              _vp, _vp, ctypes.c_size_t, _vp]),
 }
 
-ST_NONFINITE, ST_CLAMPED, ST_BAD_RANGE, ST_BAD_INDEX = 1, 2, 4, 8
+ST_NONFINITE, ST_CLAMPED, ST_BAD_RANGE, ST_BAD_INDEX, ST_OC_TRUNCATED = 1, 2, 4, 8, 16
 
 
 def lib():

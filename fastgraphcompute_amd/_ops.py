@@ -333,6 +333,116 @@ def _gravnet_aggregate_impl(idx, distsq, feat):
     return _GravNetAggregate.apply(idx, distsq, feat)
 
 
+# ------------------------------------------------------------------ object-condensation helper matrices
+def _oc_check_inputs(asso: torch.Tensor, row_splits: torch.Tensor):
+    _lib.require_device(asso, row_splits)
+    # the reference's argument checks (oc_helper_cuda_kernel.cu:118-152, oc_helper_helper.cpp:43)
+    if asso.dtype != torch.int64 or asso.dim() != 1:
+        raise RuntimeError("asso_idx should be contiguous and of type int64")
+    if row_splits.dtype != torch.int64 or row_splits.dim() != 1:
+        raise RuntimeError("row_splits must be of type int64")
+    if row_splits.numel() < 2:
+        raise RuntimeError("row_splits needs at least two entries")
+
+
+def _oc_objects(asso: torch.Tensor, row_splits: torch.Tensor, filter_negative: bool):
+    """Objects pass of the library plus the single host read the output shapes need.  Returns (workspace,
+    summary tensor, n_unique, n_maxuq, host row splits, max_per_split, objects_per_split)."""
+    L = _lib.lib()
+    dev = asso.device
+    a = asso.contiguous()
+    rs = row_splits.contiguous()
+    n, n_rs = a.numel(), rs.numel()
+    ws_bytes = L.fgc_oc_helper_workspace_bytes(n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    summary = torch.empty(4, dtype=torch.int64, device=dev)
+    max_per_split = torch.empty(n_rs - 1, dtype=torch.int64, device=dev)
+    objects_per_split = torch.empty(n_rs - 1, dtype=torch.int64, device=dev)
+    wide = 0
+    while True:
+        with torch.cuda.device(dev):
+            _lib.check(L.fgc_oc_helper_objects_i64(_lib.ptr(a), n, _lib.ptr(rs), n_rs, int(filter_negative), wide,
+                                                   _lib.ptr(max_per_split), _lib.ptr(objects_per_split),
+                                                   _lib.ptr(summary), _lib.ptr(ws), ws_bytes, _lib.stream_ptr()))
+        host = torch.cat([summary, rs]).cpu()          # the one synchronisation of the call
+        if wide == 0 and (int(host[2]) & 1):
+            wide = 1                                    # a value needs more bits than the narrow key has
+            continue
+        break
+    rs_host = host[4:]
+    if int(rs_host[0]) != 0 or int(rs_host[-1]) != n or bool((rs_host[1:] < rs_host[:-1]).any()):
+        raise ValueError("row_splits must start at 0, end at the number of vertices and not decrease")
+    return a, rs, ws, ws_bytes, summary, int(host[0]), int(host[1]), rs_host, max_per_split, objects_per_split
+
+
+def _oc_helper_matrices_impl(truth_idxs: torch.Tensor, row_splits: torch.Tensor, calc_m_not: bool):
+    if truth_idxs.device != row_splits.device:
+        raise AssertionError("Both truth_idxs and row_splits must be on the same device")
+    _oc_check_inputs(truth_idxs, row_splits)
+    L = _lib.lib()
+    a, rs, ws, ws_bytes, summary, n_unique, n_maxuq, rs_host, _mx, objects_per_split = _oc_objects(
+        truth_idxs, row_splits, True)
+    dev = a.device
+    n_maxrs = int((rs_host[1:] - rs_host[:-1]).max())
+    M = torch.empty((n_unique, n_maxuq), dtype=torch.int64, device=dev)
+    # without M_not the reference's device op hands back an empty [0, 0] tensor (oc_helper_cuda_kernel.cu:171-176)
+    M_not = torch.empty((n_unique, n_maxrs) if calc_m_not else (0, 0), dtype=torch.int64, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(L.fgc_oc_helper_fill_i64(a.numel(), _lib.ptr(rs), rs.numel(), n_unique, n_maxuq, n_maxrs, None, None,
+                                            _lib.ptr(summary), _lib.ptr(M), _lib.ptr(M_not) if calc_m_not else None,
+                                            None, None, None, _lib.ptr(ws), ws_bytes, _lib.stream_ptr()))
+    return M, M_not, objects_per_split
+
+
+def _oc_helper_cuda_impl(asso_idx: torch.Tensor, unique_idx: torch.Tensor, unique_rs_asso: torch.Tensor,
+                         rs: torch.Tensor, max_n_unique_over_splits: torch.Tensor, max_n_in_splits: torch.Tensor,
+                         calc_m_not: bool):
+    """The reference's device op (oc_helper_cuda_kernel.cu:154-203): objects and widths come from the caller."""
+    _oc_check_inputs(asso_idx, rs)
+    for t, name in ((unique_idx, "unique_idx"), (unique_rs_asso, "unique_rs_asso"),
+                    (max_n_unique_over_splits, "max_n_unique_over_splits"), (max_n_in_splits, "max_n_in_splits")):
+        if t.dtype != torch.int64 or not t.is_contiguous():
+            raise RuntimeError(name + " should be contiguous and of type int64")
+        if t.device != asso_idx.device:
+            raise RuntimeError("All inputs should be on the same device")
+    if max_n_unique_over_splits.dim() != 1 or max_n_unique_over_splits.size(0) != 1:
+        raise RuntimeError("max_n_unique_over_splits should have size 1")
+    if max_n_in_splits.dim() != 1 or max_n_in_splits.size(0) != 1:
+        raise RuntimeError("max_n_in_splits should have size 1")
+    if unique_idx.numel() != unique_rs_asso.numel() or unique_idx.numel() > max(asso_idx.numel(), 0):
+        raise RuntimeError("unique_idx and unique_rs_asso must list each object of asso_idx once")
+    L = _lib.lib()
+    dev = asso_idx.device
+    widths = torch.cat([max_n_unique_over_splits, max_n_in_splits]).cpu()
+    n_maxuq, n_maxrs = int(widths[0]), int(widths[1])
+    # negative association indices are objects too when the caller lists them
+    a, rsd, ws, ws_bytes, summary, _nu, _nm, _rs_host, _mx, _ops = _oc_objects(asso_idx, rs, False)
+    n_rows = unique_idx.numel()
+    M = torch.empty((n_rows, n_maxuq), dtype=torch.int64, device=dev)
+    M_not = torch.empty((n_rows, n_maxrs) if calc_m_not else (0, 0), dtype=torch.int64, device=dev)
+    status = torch.zeros(4, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(L.fgc_oc_helper_fill_i64(a.numel(), _lib.ptr(rsd), rsd.numel(), n_rows, n_maxuq, n_maxrs,
+                                            _lib.ptr(unique_idx), _lib.ptr(unique_rs_asso), _lib.ptr(summary),
+                                            _lib.ptr(M), _lib.ptr(M_not) if calc_m_not else None, None, None,
+                                            _lib.ptr(status), _lib.ptr(ws), ws_bytes, _lib.stream_ptr()))
+    if config.sync_checks and (int(status[0]) & _lib.ST_OC_TRUNCATED):
+        raise RuntimeError("an object has more vertices than max_n_unique_over_splits")
+    return M, M_not
+
+
+def _max_same_valued_impl(asso_idx: torch.Tensor, row_splits: torch.Tensor, filter_negative: bool):
+    """max_same_valued_entries_per_row_split (oc_helper_helper.cpp:30-94); row_splits may live on the host as in
+    the reference, the results are on asso_idx's device."""
+    if row_splits.dtype != torch.int64:
+        raise RuntimeError("row_splits must be of type int64")
+    rs = row_splits.to(asso_idx.device)
+    _oc_check_inputs(asso_idx, rs)
+    out = _oc_objects(asso_idx, rs, filter_negative)
+    max_per_split, objects_per_split = out[8], out[9]
+    return max_per_split, max_per_split.max(), objects_per_split
+
+
 # ------------------------------------------------------------------ registration
 def _register():
     lib = _define("bin_by_coordinates",
@@ -359,6 +469,20 @@ def _register():
     lib.impl("gravnet_aggregate", _gravnet_aggregate_impl, "Autograd")
     lib.define("select_with_default_f32(Tensor idx, Tensor feat, float default_value) -> Tensor")
     lib.impl("select_with_default_f32", _select_with_default_impl, "Autograd")
+
+    lib = _define("oc_helper_cuda",
+                  "oc_helper_cuda(Tensor asso_idx, Tensor unique_idx, Tensor unique_rs_asso, Tensor rs, "
+                  "Tensor max_n_unique_over_splits, Tensor max_n_in_splits, bool calc_m_not) -> (Tensor, Tensor)")
+    lib.impl("oc_helper_cuda", _oc_helper_cuda_impl, "CUDA")
+    lib.impl("oc_helper_cuda", _oc_helper_cuda_impl, "CPU")
+    lib.define("oc_helper_matrices(Tensor truth_idxs, Tensor row_splits, bool calc_m_not) -> "
+               "(Tensor, Tensor, Tensor)")
+    lib.impl("oc_helper_matrices", _oc_helper_matrices_impl, "CUDA")
+    lib.impl("oc_helper_matrices", _oc_helper_matrices_impl, "CPU")
+    lib.define("max_same_valued_entries_per_row_split(Tensor asso_idx, Tensor row_splits, bool filter_negative) "
+               "-> (Tensor, Tensor, Tensor)")
+    lib.impl("max_same_valued_entries_per_row_split", _max_same_valued_impl, "CUDA")
+    lib.impl("max_same_valued_entries_per_row_split", _max_same_valued_impl, "CPU")
 
 
 _register()

@@ -481,11 +481,11 @@ size_t fgc_sort_workspace_bytes(int64_t n)
            fgc_align(256 * 4) /* digit totals */;
 }
 
-// Sorts (keys, identity) stably by the low `key_bits` bits.  On return
-// *keys_sorted / *vals_sorted point at the buffers holding the result
+// Sorts (keys, vals) stably by the low `key_bits` bits; vals start as the identity unless
+// `vals_given`.  On return *keys_sorted / *vals_sorted point at the buffers holding the result
 // (either the caller's primary pair or the alternates inside the workspace).
 int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void *d_ws, hipStream_t s,
-                  uint32_t **keys_sorted, uint32_t **vals_sorted)
+                  uint32_t **keys_sorted, uint32_t **vals_sorted, bool vals_given)
 {
     if (n >= (1ll << 31)) return FGC_EINVAL;
     char *w = (char *)d_ws;
@@ -495,7 +495,7 @@ int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void 
     int nblk = (int)fgc_cdiv(n, RS_TILE);
     uint32_t *digit_total = (uint32_t *)(w + fgc_align((size_t)nblk * 256 * 4));
     if ((int64_t)nblk * 256 >= (1ll << 31)) return FGC_EINVAL;
-    uint32_t *kin = keys, *vin = nullptr, *kout = k_alt, *vout = v_alt;
+    uint32_t *kin = keys, *vin = vals_given ? vals : nullptr, *kout = k_alt, *vout = v_alt;
     int passes = (key_bits + 7) / 8;
     if (passes < 1) passes = 1;
     for (int p = 0; p < passes; p++) {

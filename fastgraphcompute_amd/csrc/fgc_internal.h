@@ -4,7 +4,7 @@
 
 size_t fgc_sort_workspace_bytes(int64_t n);
 int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void *d_ws, hipStream_t s,
-                  uint32_t **keys_sorted, uint32_t **vals_sorted);
+                  uint32_t **keys_sorted, uint32_t **vals_sorted, bool vals_given = false);
 int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, int sub_bits, const float *d_geom,
                         const int64_t *d_rs, int n_rs, uint32_t *d_keys, int *d_status, hipStream_t s);
 int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int shift, int n_bins_total, int *bb, hipStream_t s);

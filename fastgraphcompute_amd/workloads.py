@@ -87,3 +87,22 @@ CONFIGS = {
     "cfg4": cfg4_zipf_blobs,
     "cfg5": cfg5_many_events_d8,
 }
+
+
+def oc_workload(scale=1.0):
+    """Truth indices for the object-condensation helper: 4 events of 50 000 vertices, 500 objects per event with
+    sizes ~ rank^-1 (a few large showers, many small ones), 10 % noise vertices (-1), shuffled inside the event;
+    object ids restart at 0 in every event.  Returns (int64 truth indices [200 000], int64 row_splits [5])."""
+    rng = np.random.default_rng(1006)
+    per_event = int(round(50000 * scale))
+    n_obj = 500
+    p = 1.0 / np.arange(1, n_obj + 1)
+    p /= p.sum()
+    parts = []
+    for _ in range(4):
+        t = rng.choice(n_obj, size=per_event, p=p)
+        t[rng.random(per_event) < 0.1] = -1
+        parts.append(t)
+    a = np.concatenate(parts).astype(np.int64)
+    rs = (np.arange(5) * per_event).astype(np.int64)
+    return a, rs

@@ -41,6 +41,7 @@ extern "C" {
 #define FGC_ST_CLAMPED 2     /* a coordinate fell outside the grid (clamped)  */
 #define FGC_ST_BAD_RANGE 4   /* range / bin width / n_bins not positive       */
 #define FGC_ST_BAD_INDEX 8   /* neighbour index >= n_vert seen (gradient)     */
+#define FGC_ST_OC_TRUNCATED 16 /* an object has more vertices than M is wide   */
 
 /* Library version (major*100 + minor) and the text for a return code. */
 int fgc_version(void);
@@ -201,6 +202,64 @@ int fgc_gravnet_aggregate_bwd_f32(const int64_t *d_idx, const float *d_distsq,
                                   const float *d_grad_fmean, const float *d_grad_fmax,
                                   float *d_grad_feat, float *d_grad_distsq, int64_t n_vert,
                                   int32_t K, int32_t P, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Object-condensation helper matrices.  Two calls with one host read between
+ * them (the output shapes depend on the data):
+ *
+ * fgc_oc_helper_objects_i64 replaces the input analysis of oc_helper_matrices,
+ * i.e. _helper_inputs (oc_helper.py:18-149: torch.unique over (value, row
+ * split) pairs) and max_same_valued_entries_per_row_split
+ * (oc_helper_helper.cpp:30-94).  An object is a distinct (association index,
+ * row split) pair; with filter_negative != 0 negative indices form no object.
+ *   d_asso               int64 [n_vert] association (truth) index per vertex
+ *   d_row_splits         int64 [n_rs] on the device
+ *   wide_keys            0: sort on 32-bit keys (row split beside value + 1);
+ *                        summary[2] bit 0 is set when a value does not fit and
+ *                        the call must be repeated with wide_keys = 1 (full
+ *                        64-bit values, three sorts).  Forced when
+ *                        filter_negative == 0.
+ *   d_max_per_split      out int64 [n_rs-1] vertices of the largest object
+ *   d_objects_per_split  out int64 [n_rs-1] number of objects
+ *   d_summary            out int64 [FGC_OC_SUMMARY_WORDS]: [0] number of objects
+ *                        (rows of M), [1] vertices of the largest object
+ *                        (columns of M), [2] flags
+ *   d_ws                 fgc_oc_helper_workspace_bytes(n_vert) bytes; holds the
+ *                        object table (ordered by row split, then value) that
+ *                        fgc_oc_helper_fill_i64 reads
+ *
+ * fgc_oc_helper_fill_i64 replaces oc_helper_cuda_fn
+ * (oc_helper_cuda_kernel.cu:154-203, kernel calc_m :19-116; CPU twin
+ * oc_helper_cpu.cpp:17-82) including its transposes: row k of M [n_rows,
+ * n_maxuq] lists the vertices of object k in ascending order, row k of M_not
+ * [n_rows, n_maxrs] the other vertices of the object's row split in ascending
+ * order, both padded with -1.
+ *   d_unique_idx, d_unique_rs  NULL: rows follow the library's object table
+ *                        (n_rows = summary[0]); else int64 [n_rows] objects in
+ *                        the caller's order as the reference's op takes them
+ *                        (a pair without vertices gives an all -1 row of M and
+ *                        the whole row split in M_not); d_summary is then read
+ *                        on the device
+ *   d_M_not              NULL to skip (calc_m_not = False)
+ *   d_obj_idx_out, d_obj_rs_out  optional int64 [n_rows]: value and row split
+ *                        of each object of the library's table
+ *   d_status             optional int32[FGC_STATUS_WORDS]; FGC_ST_OC_TRUNCATED
+ *                        when n_maxuq is smaller than an object (the reference
+ *                        prints and stops filling, oc_helper_cuda_kernel.cu:59-63)
+ * Row splits longer than n_maxrs are cut to n_maxrs vertices as in
+ * oc_helper_cuda_kernel.cu:49-52.
+ */
+#define FGC_OC_SUMMARY_WORDS 4
+size_t fgc_oc_helper_workspace_bytes(int64_t n_vert);
+int fgc_oc_helper_objects_i64(const int64_t *d_asso, int64_t n_vert, const int64_t *d_row_splits, int32_t n_rs,
+                              int32_t filter_negative, int32_t wide_keys, int64_t *d_max_per_split,
+                              int64_t *d_objects_per_split, int64_t *d_summary, void *d_ws, size_t ws_bytes,
+                              void *stream);
+int fgc_oc_helper_fill_i64(int64_t n_vert, const int64_t *d_row_splits, int32_t n_rs, int64_t n_rows,
+                           int64_t n_maxuq, int64_t n_maxrs, const int64_t *d_unique_idx,
+                           const int64_t *d_unique_rs, const int64_t *d_summary, int64_t *d_M, int64_t *d_M_not,
+                           int64_t *d_obj_idx_out, int64_t *d_obj_rs_out, int32_t *d_status, const void *d_ws,
+                           size_t ws_bytes, void *stream);
 
 #ifdef __cplusplus
 }

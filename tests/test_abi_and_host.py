@@ -65,8 +65,11 @@ def test_host_wrappers_reject_cpu_tensors_and_bad_arguments():
         fgc.bin_by_coordinates(torch.rand(10, 3), torch.tensor([0, 10]), n_bins=4)
     with pytest.raises((AssertionError, RuntimeError, torch.jit.Error)):
         fgc.index_replacer(torch.zeros(3, dtype=torch.int32), torch.zeros(3, dtype=torch.int64))
-    with pytest.raises(NotImplementedError):
-        fgc.oc_helper_matrices()
+    with pytest.raises((RuntimeError, torch.jit.Error)):          # no CPU fallback
+        fgc.oc_helper_matrices(torch.tensor([1, 1, 2]), torch.tensor([0, 3]))
+    with pytest.raises(RuntimeError):
+        fgc.extensions.oc_helper.max_same_valued_entries_per_row_split(torch.tensor([1, 1, 2]), torch.tensor([0, 3]),
+                                                                       True)
 
 
 def test_n_bins_heuristic_host():
