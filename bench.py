@@ -30,7 +30,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "oc_helper"])
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seconds", type=float, default=15.0)
@@ -54,6 +54,8 @@ def main():
     torch.cuda.set_device(dev)
     L = _lib.lib()
 
+    if args.workload == "oc_helper":
+        return oc_helper_workload(args, dev)
     w = workloads.CONFIGS[args.workload](args.scale)
     if args.workload == "cfg3":
         return gravnet_workload(args, w, dev)
@@ -194,6 +196,88 @@ def gravnet_workload(args, w, dev):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(t * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": w["name"], "n_points": n, "events": 2}}), flush=True)
+
+
+def oc_helper_workload(args, dev):
+    """Secondary workload: oc_helper_matrices on 200 000 vertices in 4 events with 500 objects each (M_not is
+    [2000, 50000] int64 = 800 MB).  The roofline entry is the M_not kernel's HBM write stream."""
+    import numpy as np
+    import torch
+    import fastgraphcompute_amd as fgc
+    from fastgraphcompute_amd import _lib, workloads
+    L = _lib.lib()
+    a_h, rs_h = workloads.oc_workload(args.scale)
+    a = torch.from_numpy(a_h).to(dev)
+    rs = torch.from_numpy(rs_h).to(dev)
+
+    def step():
+        return fgc.oc_helper_matrices(a, rs)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        M, M_not, _n = step()
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / args.steps
+
+    # the two library calls on their own, timed with events on the stream they are enqueued on
+    n, n_rs = a.numel(), rs.numel()
+    ws_bytes = L.fgc_oc_helper_workspace_bytes(n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    summary = torch.empty(4, dtype=torch.int64, device=dev)
+    mx = torch.empty(n_rs - 1, dtype=torch.int64, device=dev)
+    no = torch.empty_like(mx)
+    U, W, R = M.shape[0], M.shape[1], M_not.shape[1]
+
+    def objects():
+        _lib.check(L.fgc_oc_helper_objects_i64(_lib.ptr(a), n, _lib.ptr(rs), n_rs, 1, 0, _lib.ptr(mx), _lib.ptr(no),
+                                               _lib.ptr(summary), _lib.ptr(ws), ws_bytes, _lib.stream_ptr()))
+
+    def fill(m, m_not):
+        _lib.check(L.fgc_oc_helper_fill_i64(n, _lib.ptr(rs), n_rs, U, W, R, None, None, _lib.ptr(summary),
+                                            _lib.ptr(M) if m else None, _lib.ptr(M_not) if m_not else None, None,
+                                            None, None, _lib.ptr(ws), ws_bytes, _lib.stream_ptr()))
+
+    def timed(fn, reps=20):
+        fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e-3
+
+    t_obj = timed(objects)
+    t_m = timed(lambda: fill(True, False))
+    t_not = timed(lambda: fill(False, True))
+    bytes_not = 8.0 * U * R + 4.0 * n                # every int64 written once + one read of the object ids
+    result = {
+        "metric": "oc_helper_matrices vertices/sec", "value": round(n / t, 1), "unit": "vertices/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(t * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int64", "data": "synthetic",
+        "config": {"workload": "oc_helper_200k_4events_500objects", "n_vertices": n, "events": int(n_rs - 1),
+                   "n_objects": int(U), "M_columns": int(W), "M_not_columns": int(R)},
+        "stages_ms": {"objects": round(t_obj * 1e3, 4), "fill_M": round(t_m * 1e3, 4),
+                      "fill_M_not": round(t_not * 1e3, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(bytes_not / t_not / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
+                     "frac": round(bytes_not / t_not / 8e12, 4), "traffic": None, "kernel": "k_oc_fill_m_not"},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import oracle as O
+        uv, ur, gmax, _l, max_len, _nobj = O.oc_helper_inputs(a_h, rs_h, True)
+        sel = np.arange(uv.size)
+        O.oc_calc_m(a_h, uv[:8], ur[:8], rs_h, gmax, max_len, True)     # page in the library
+        t0 = time.perf_counter()
+        for _ in range(3):
+            O.oc_calc_m(a_h, uv, ur, rs_h, gmax, max_len, True)
+        tc = (time.perf_counter() - t0) / 3
+        result["cpu_baseline"] = {"value": round(n * (sel.size / uv.size) / tc, 1), "unit": "vertices/s", "cores": 1,
+                                  "kind": "port", "sample": "calc_m restatement on %d of %d objects (%.2f s per pass, 3 passes), "
+                                  "object analysis excluded" % (sel.size, uv.size, tc)}
+    print(json.dumps(result), flush=True)
 
 
 def cpu_baseline(w, K, n, budget_s):

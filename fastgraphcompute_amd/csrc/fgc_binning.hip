@@ -422,12 +422,22 @@ __global__ __launch_bounds__(256) void k_rs_scatter(const uint32_t *__restrict__
             uint32_t u = __shfl_up(incl, o, 64);
             if (ln >= o) incl += u;
         }
+        __shared__ int s_const;
+        if (t == 0) s_const = 0;
         if (ln == 63) s_ws[w] = incl;
         __syncthreads();
         uint32_t off = 0;
         for (int k = 0; k < w; k++) off += s_ws[k];
         s_dig[t] = off + incl - v;
+        if (v == (uint32_t)n) s_const = 1;      // every key has this digit: the pass is the identity
         __syncthreads();
+        if (s_const) {
+            for (int i = blockIdx.x * RS_TILE + t; i < min(n, (int)(blockIdx.x + 1) * RS_TILE); i += 256) {
+                keys_out[i] = keys_in[i];
+                vals_out[i] = vals_in ? vals_in[i] : (uint32_t)i;
+            }
+            return;
+        }
     }
     const int lane = fgc_lane(), wv = threadIdx.x >> 6;
     volatile uint32_t *cnt = s_cnt[wv];

@@ -14,8 +14,15 @@
 namespace {
 
 constexpr int OC_BLOCK = 256;
-constexpr int OC_NOT_CHUNK = 4096;                 // vertex offsets of one row handled by one block
+#ifndef FGC_OC_NOT_CHUNK
+#define FGC_OC_NOT_CHUNK 4096
+#endif
+constexpr int OC_NOT_CHUNK = FGC_OC_NOT_CHUNK;     // vertex offsets of one row handled by one block
 constexpr int OC_NOT_WAVE = OC_NOT_CHUNK / 4;      // ... by one wavefront
+#ifndef FGC_OC_FEW
+#define FGC_OC_FEW 16
+#endif
+constexpr int OC_FEW = FGC_OC_FEW;                 // members per slice up to which gaps are computed, not compacted
 enum { OC_KEY_NARROW = 0, OC_KEY_LO = 1, OC_KEY_HI = 2, OC_KEY_RS = 3 };
 
 // summary record (int64 words)
@@ -263,6 +270,25 @@ __device__ __forceinline__ int oc_rank_below(const uint32_t *__restrict__ mem, i
     return lo;
 }
 
+// dst[j] = value(j) for j in [0, count) by one wavefront: a single 8-byte store brings dst to a 16-byte
+// boundary, then every lane stores two elements at a time
+template <class F>
+__device__ __forceinline__ void oc_stream_out(int64_t *__restrict__ dst, int count, int lane, F value)
+{
+    if (count <= 0) return;
+    const int head = (int)(((uintptr_t)dst >> 3) & 1);
+    if (head && lane == 0) dst[0] = value(0);
+    const int pairs = (count - head) >> 1;
+    longlong2 *d2 = (longlong2 *)(dst + head);
+    for (int j = lane; j < pairs; j += 64) {
+        longlong2 v;
+        v.x = value(head + 2 * j);
+        v.y = value(head + 2 * j + 1);
+        d2[j] = v;
+    }
+    if (((count - head) & 1) && lane == 63) dst[count - 1] = value(count - 1);
+}
+
 // M_not: for block (row, chunk) the vertex offsets [chunk * OC_NOT_CHUNK, +OC_NOT_CHUNK) of the row's split,
 // compacted to the vertices outside the object, plus the -1 padding that falls into the same output range.
 __global__ __launch_bounds__(OC_BLOCK) void k_oc_fill_m_not(const uint32_t *__restrict__ perm,
@@ -275,8 +301,10 @@ __global__ __launch_bounds__(OC_BLOCK) void k_oc_fill_m_not(const uint32_t *__re
                                                             const int64_t *__restrict__ rs, int n_rs, int n_vert,
                                                             int n_chunks, int n_maxrs, int64_t *__restrict__ M_not)
 {
+    __shared__ int s_buf[4][OC_NOT_WAVE];
     const int row = blockIdx.x / n_chunks, chunk = blockIdx.x - row * n_chunks;
     const int lane = fgc_lane(), wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    int *buf = s_buf[wv];
     const int k = map ? map[row] : row;
     int r;
     if (q_rs) {
@@ -300,22 +328,50 @@ __global__ __launch_bounds__(OC_BLOCK) void k_oc_fill_m_not(const uint32_t *__re
     const int o0 = chunk * OC_NOT_CHUNK + wv * OC_NOT_WAVE;
     const int o1 = min(o0 + OC_NOT_WAVE, len);
     if (o0 < len) {
-        int base = o0 - (cnt > 0 ? oc_rank_below(mem, cnt, (uint32_t)(lo + o0)) : 0);
-        for (int g = o0; g < o1; g += 256) {
-            int id[4];
+        // members of the object below the slice (r0) and below its end (r1)
+        int r0 = 0, r1 = 0;
+        uint32_t mine = 0xffffffffu;                 // member r0 + lane when the slice holds at most 64 of them
+        if (cnt > 0 && cnt <= 64) {
+            const uint32_t v = lane < cnt ? mem[lane] : 0xffffffffu;
+            r0 = __popcll(fgc_ballot(v < (uint32_t)(lo + o0)));
+            r1 = __popcll(fgc_ballot(v < (uint32_t)(lo + o1)));
+            mine = (uint32_t)__shfl((int)v, (r0 + lane) & 63, 64);
+            if (lane >= r1 - r0) mine = 0xffffffffu;
+        } else if (cnt > 64) {
+            r0 = oc_rank_below(mem, cnt, (uint32_t)(lo + o0));
+            r1 = r0 + oc_rank_below(mem + r0, min(cnt - r0, OC_NOT_WAVE), (uint32_t)(lo + o1));
+            if (r1 - r0 <= OC_FEW && lane < r1 - r0) mine = mem[r0 + lane];
+        }
+        const int base = o0 - r0, in_slice = r1 - r0, kept = (o1 - o0) - in_slice;
+        if (in_slice <= OC_FEW) {
+            // few gaps: element j of the output is offset o0 + j + (members that come before it); member i
+            // comes before element j when the kept vertices in front of it, d_i, number at most j
+            const int d = mine == 0xffffffffu ? 0x7fffffff : (int)mine - lo - o0 - lane;
+            oc_stream_out(out + base, kept, lane, [&](int j) {
+                int t = 0;
+                for (int i = 0; i < in_slice; i++) t += (fgc_readlane_i(d, i) <= j) ? 1 : 0;
+                return (int64_t)(lo + o0 + j + t);
+            });
+        } else {
+            // many gaps: compact the kept vertices in LDS by ballots over the object id of every vertex
+            int pos = 0;
+            for (int g = o0; g < o1; g += 256) {
+                int id[4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int off = g + u * 64 + lane;
-                id[u] = off < o1 ? oid[lo + off] : k;
-            }
+                for (int u = 0; u < 4; u++) {
+                    const int off = g + u * 64 + lane;
+                    id[u] = off < o1 ? oid[lo + off] : k;
+                }
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int off = g + u * 64 + lane;
-                const bool keep = off < o1 && (k < 0 || id[u] != k);
-                const unsigned long long m = fgc_ballot(keep);
-                if (keep) out[base + fgc_mbcnt(m)] = (int64_t)(lo + off);
-                base += __popcll(m);
+                for (int u = 0; u < 4; u++) {
+                    const int off = g + u * 64 + lane;
+                    const bool keep = off < o1 && id[u] != k;
+                    const unsigned long long m = fgc_ballot(keep);
+                    if (keep) buf[pos + fgc_mbcnt(m)] = lo + off;
+                    pos += __popcll(m);
+                }
             }
+            oc_stream_out(out + base, pos, lane, [&](int j) { return (int64_t)buf[j]; });
         }
     }
     // padding positions inside this wavefront's output range
@@ -324,7 +380,7 @@ __global__ __launch_bounds__(OC_BLOCK) void k_oc_fill_m_not(const uint32_t *__re
         int members = cnt;
         if (clipped && cnt > 0) members = oc_rank_below(mem, cnt, (uint32_t)(lo + len));
         const int pad0 = max(o0, len - members);
-        for (int p = pad0 + lane; p < e1; p += 64) out[p] = -1;
+        oc_stream_out(out + pad0, e1 - pad0, lane, [](int) { return (int64_t)-1; });
     }
 }
 
