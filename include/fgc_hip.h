@@ -110,7 +110,7 @@ int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t ld_coords,
  *                 fewer than K points
  *   d_distsq      out float32 [n_vert, K], 0 for slot 0 and for padding
  *   d_stats       optional uint64[4] device counters, accumulated: [0] distance
- *                 evaluations, [1] candidate chunks visited, [2] insertions;
+ *                 evaluations, [1] candidate chunks visited, [2] pool prunes;
  *                 NULL to skip
  */
 size_t fgc_binned_select_knn_workspace_bytes(int64_t n_vert, int32_t n_coords,
