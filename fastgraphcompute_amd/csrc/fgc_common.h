@@ -58,6 +58,16 @@ __device__ __forceinline__ float fgc_wave_sum(float v)
     return (fgc_readlane_f(v, 0) + fgc_readlane_f(v, 16)) + (fgc_readlane_f(v, 32) + fgc_readlane_f(v, 48));
 }
 
+// maximum of v over the 64 lanes (returned in every lane), same data movement as fgc_wave_sum
+__device__ __forceinline__ int fgc_wave_max_i(int v)
+{
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x140, 0xf, 0xf, true));
+    return max(max(fgc_readlane_i(v, 0), fgc_readlane_i(v, 16)), max(fgc_readlane_i(v, 32), fgc_readlane_i(v, 48)));
+}
+
 // internal launchers shared between translation units (all enqueue on `s`)
 int fgc_fill_u32(void *d, uint32_t v, int64_t n_words, hipStream_t s);
 int fgc_copy_u32(void *dst, const void *src, int64_t n_words, hipStream_t s);

@@ -145,7 +145,13 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             for (int s = 0; s < PS; s++) n += __popcll(fgc_ballot(P[s] <= t));
             return n;
         };
-        const float told = fgc_readlane_f(tau, q);
+        float told = fgc_readlane_f(tau, q);
+        if (!(told < INFINITY)) {              // first fill: bracket by the largest distance in the pool
+            int mx = 0;
+#pragma unroll
+            for (int s = 0; s < PS; s++) mx = max(mx, P[s] == 0xffffffffu ? 0 : (int)P[s]);
+            told = __int_as_float(fgc_wave_max_i(mx));
+        }
         unsigned hi = (told < INFINITY) ? __float_as_uint(told) : 0x7f7fffffu;   // count_le(hi) >= K
         int chi = c;
         bool converged = false;
@@ -411,43 +417,30 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                         TM_STOP(tm_eval);
                         if (!pm) continue;
                         TM_START();
-                        // ---- append the passing lanes to query q's pool, pruning when it runs full: first to
-                        //      a tighter threshold, then (if that is not enough) down to exactly K ----
+                        // ---- append the passing lanes to query q's pool; when it overflows or runs nearly
+                        //      full (tau should stay tight) prune it: first to a tighter threshold, then, if
+                        //      lanes are still waiting, down to exactly K ----
                         int pc = fgc_readlane_i(cnt, q);
-                        if (__popcll(pm) <= CAP - pc) {
-                            if ((pm >> lane) & 1ull) {
-                                const int pos = pc + fgc_mbcnt(pm);
-                                ld[q * CAP + pos] = dsq;
-                                li[q * CAP + pos] = j;
+                        for (int attempt = 0;; attempt++) {
+                            const int room = CAP - pc;
+                            const int rnk = fgc_mbcnt(pm);
+                            const bool put = ((pm >> lane) & 1ull) && rnk < room;
+                            if (put) {
+                                ld[q * CAP + pc + rnk] = dsq;
+                                li[q * CAP + pc + rnk] = j;
                             }
-                            pc += __popcll(pm);
+                            const int npm = __popcll(pm);
+                            pc += min(npm, room);
                             cnt = (lane == q) ? pc : cnt;
-                        } else {
-                            int attempt = 0;
-                            while (pm) {
-                                int room = CAP - pc;
-                                if (__popcll(pm) > room) {
-                                    prune(q, attempt > 0);
-                                    attempt++;
-                                    pm &= fgc_ballot(dsq < fgc_readlane_f(tau, q));
-                                    pc = fgc_readlane_i(cnt, q);
-                                    room = CAP - pc;
-                                    if (!pm) break;
-                                }
-                                const int rnk = fgc_mbcnt(pm);
-                                const bool put = ((pm >> lane) & 1ull) && rnk < room;
-                                const unsigned long long sub = fgc_ballot(put);
-                                if (put) {
-                                    ld[q * CAP + pc + rnk] = dsq;
-                                    li[q * CAP + pc + rnk] = j;
-                                }
-                                pc += __popcll(sub);
-                                cnt = (lane == q) ? pc : cnt;
-                                pm &= ~sub;
-                            }
+                            const bool left = npm > room;          // lanes of rank >= room are still waiting
+                            if (!left && pc <= CAP - PRUNE_MARGIN && (pc <= K || fgc_readlane_f(tau, q) < INFINITY))
+                                break;
+                            prune(q, attempt > 0);
+                            if (!left) break;
+                            pc = fgc_readlane_i(cnt, q);
+                            pm = fgc_ballot(((pm >> lane) & 1ull) && rnk >= room && dsq < fgc_readlane_f(tau, q));
+                            if (!pm) break;
                         }
-                        // keep tau tight: prune as soon as the pool is nearly full
-                        if (pc > CAP - PRUNE_MARGIN || (pc > K && !(fgc_readlane_f(tau, q) < INFINITY))) prune(q, false);
                         TM_STOP(tm_pool);
                     }
                 }
