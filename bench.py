@@ -30,7 +30,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "oc_helper"])
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "oc_helper", "gravnet_model"])
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seconds", type=float, default=15.0)
@@ -46,6 +46,7 @@ def main():
     from fastgraphcompute_amd import _lib, config, workloads
     from fastgraphcompute_amd.extensions.binned_select_knn import (binned_select_knn_grad,
                                                                    calculate_optimal_bins)
+    from fastgraphcompute_amd._ops import choose_search_grid
 
     if not torch.cuda.is_available():
         print("bench.py: no HIP device visible", file=sys.stderr)
@@ -56,6 +57,8 @@ def main():
 
     if args.workload == "oc_helper":
         return oc_helper_workload(args, dev)
+    if args.workload == "gravnet_model":
+        return gravnet_model_workload(args, dev)
     w = workloads.CONFIGS[args.workload](args.scale)
     if args.workload == "cfg3":
         return gravnet_workload(args, w, dev)
@@ -91,8 +94,12 @@ def main():
 
     # ---- stage timings with events on the launch stream (torch's current stream) ----
     rs_host = rs.cpu()
-    nbd = min(3, D)
-    nb = [calculate_optimal_bins(rs_host, K, nbd)] * nbd
+    if config.auto_grid:                       # the grid binned_select_knn itself picks when n_bins is None
+        nbd, nb1 = choose_search_grid(rs_host, D, 3)
+        nb = [nb1] * nbd
+    else:
+        nbd = min(3, D)
+        nb = [calculate_optimal_bins(rs_host, K, nbd)] * nbd
     nb_arr, rs_arr = _lib.host_i64(nb), _lib.host_i64(rs_host.tolist())
     n_rs = rs_host.numel()
     ws_bytes = L.fgc_binned_select_knn_workspace_bytes(n, D, nbd, nb_arr, n_rs, K)
@@ -196,6 +203,64 @@ def gravnet_workload(args, w, dev):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(t * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": w["name"], "n_points": n, "events": 2}}), flush=True)
+
+
+def gravnet_model_workload(args, dev):
+    """Secondary workload: the training step of the reference's model benchmark (performance/gravnet_perfm.py:
+    20-96,110-163): two dense layers, 4 x (GravNetOp(k=64, S=4, P=32) + three dense layers), two dense layers;
+    hidden 128, 200 000 nodes in one event, loss = sum(output) * 0, SGD step."""
+    import torch
+    import torch.nn as nn
+    from fastgraphcompute_amd.gnn_ops import GravNetOp
+
+    in_dim, prop_dim, space_dim, k, hidden, out_dim, layers = 64, 32, 4, 64, 128, 10, 4
+
+    class GravNetModel(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc1 = nn.Linear(in_dim, hidden)
+            self.fc2 = nn.Linear(hidden, hidden)
+            self.gravnet_layers = nn.ModuleList(
+                GravNetOp(hidden if i == 0 else 2 * prop_dim, 2 * prop_dim, space_dim, prop_dim, k)
+                for i in range(layers))
+            self.dense_after_gravnet = nn.ModuleList(
+                nn.Sequential(nn.Linear(2 * prop_dim, hidden), nn.ReLU(), nn.Linear(hidden, hidden), nn.ReLU(),
+                              nn.Linear(hidden, 2 * prop_dim), nn.ReLU()) for _ in range(layers))
+            self.fc3 = nn.Linear(2 * prop_dim, hidden)
+            self.fc4 = nn.Linear(hidden, out_dim)
+
+        def forward(self, x, row_splits):
+            x = torch.relu(self.fc2(torch.relu(self.fc1(x))))
+            for g, d in zip(self.gravnet_layers, self.dense_after_gravnet):
+                x = d(g(x, row_splits)[0])
+            return self.fc4(torch.relu(self.fc3(x)))
+
+    n = int(round(200000 * args.scale))
+    torch.manual_seed(1007)
+    model = GravNetModel().to(dev)
+    opt = torch.optim.SGD(model.parameters(), lr=0.01)
+    x = torch.randn(n, in_dim, device=dev)
+    rs = torch.tensor([0, n], dtype=torch.int64, device=dev)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        out = model(x, rs)
+        (out.sum() * 0.0).backward()
+        opt.step()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / args.steps
+    print(json.dumps({
+        "metric": "GravNet model training step nodes/sec", "value": round(n / t, 1), "unit": "nodes/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(t * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "gravnet_model_4layers_h128_k64", "n_points": n, "events": 1}}), flush=True)
 
 
 def oc_helper_workload(args, dev):

@@ -8,3 +8,8 @@ sync_checks = True
 # Accumulate the kNN kernel's counters (distance evaluations, candidate chunks,
 # list insertions) into binned_select_knn.last_stats; used by the benchmark.
 collect_stats = False
+
+# When binned_select_knn is called without n_bins, size the search grid for this library's search (coarse bins
+# over up to four dimensions) instead of with the reference's heuristic and max_bin_dims.  The neighbours
+# returned are the same either way; only the run time differs.
+auto_grid = True

@@ -20,7 +20,7 @@ extern "C" const char *fgc_error_string(int code)
 
 namespace {
 struct KnnWorkspace {
-    size_t geom, partial, keys, vals, sort, sort_alt_vals, bb, sc, sdir, box_lo, box_hi, total;
+    size_t geom, partial, keys, vals, sort, sort_alt_vals, bb, sc, sdir, box_lo, box_hi, sbox_lo, sbox_hi, total;
     int ldc;
 };
 
@@ -54,6 +54,8 @@ KnnWorkspace plan(int64_t n, int D, int nbd, const int64_t *n_bins, int n_rs, bo
     w.sdir = take(with_dir ? (size_t)n : 0);
     w.box_lo = take((size_t)(w.ldc / 64) * D * 4);
     w.box_hi = take((size_t)(w.ldc / 64) * D * 4);
+    w.sbox_lo = take((size_t)((w.ldc / 64 + 63) / 64) * D * 4);
+    w.sbox_hi = take((size_t)((w.ldc / 64 + 63) / 64) * D * 4);
     w.total = off;
     return w;
 }
@@ -142,7 +144,7 @@ extern "C" int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert,
     float *sc = (float *)(ws + w.sc);
     unsigned char *sdir = d_direction ? (unsigned char *)(ws + w.sdir) : nullptr;
 
-    rc = fgc_bin_geometry_f32(d_coords, n_vert, n_coords, n_bin_dims, 0, n_bins, 1, 0.f, 0, geom, d_status,
+    rc = fgc_bin_geometry_f32(d_coords, n_vert, n_coords, n_bin_dims, 2, n_bins, 1, 0.f, 0, geom, d_status,
                               ws + w.partial, fgc_bin_geometry_workspace_bytes(n_vert), stream);
     if (rc) return rc;
     rc = fgc_launch_bin_keys(d_coords, (int)n_vert, n_coords, n_bin_dims, c.sub_bits, geom, d_row_splits, n_rs,
@@ -159,7 +161,7 @@ extern "C" int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert,
     rc = fgc_launch_gather_sorted(d_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir, s);
     if (rc) return rc;
     return fgc_launch_chunk_boxes(sc, (int)n_vert, n_coords, w.ldc, (float *)(ws + w.box_lo),
-                                  (float *)(ws + w.box_hi), s);
+                                  (float *)(ws + w.box_hi), (float *)(ws + w.sbox_lo), (float *)(ws + w.sbox_hi), s);
 }
 
 extern "C" int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
@@ -182,6 +184,8 @@ extern "C" int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const
     a.key_shift = c.sub_bits * n_bin_dims;
     a.box_lo = (const float *)(ws + c.w.box_lo); a.box_hi = (const float *)(ws + c.w.box_hi);
     a.n_chunks = c.w.ldc / 64;
+    a.sbox_lo = (const float *)(ws + c.w.sbox_lo); a.sbox_hi = (const float *)(ws + c.w.sbox_hi);
+    a.n_super = (a.n_chunks + 63) / 64;
     a.bb = (const int *)(ws + c.w.bb); a.geom = (const float *)(ws + c.w.geom);
     a.sdir = with_direction ? (const unsigned char *)(ws + c.w.sdir) : nullptr;
     a.n = (int)n_vert; a.D = n_coords; a.nbd = n_bin_dims; a.K = K; a.tf_compat = tf_compat;

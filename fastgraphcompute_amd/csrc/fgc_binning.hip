@@ -133,14 +133,16 @@ __global__ __launch_bounds__(64) void k_geometry(const float *__restrict__ parti
         float lo = pre_norm ? mn[d] : (mn[d] - sub);
         float hi = pre_norm ? mx[d] : (mx[d] - sub);
         if (lo == hi) hi = hi + 1.0f;
-        hi = hi + 1e-3f;
+        // mode 2 (the kNN search's own grid) pads the range relatively: point clouds that are tiny in absolute
+        // terms still spread over all bins
+        hi = (mode == 2) ? lo + (hi - lo) * 1.001f : hi + 1e-3f;
         if (!isfinite(hi)) hi = 1.0f;
         if (!(hi > 0.f)) flags |= FGC_ST_BAD_RANGE;
         rng[d] = hi;
         geom[FGC_GEOM_MIN + d] = sub;
     }
     int nbo[FGC_MAX_BIN_DIMS] = {1, 1, 1, 1, 1};
-    if (mode == 0) {
+    if (mode == 0 || mode == 2) {
         float w = -INFINITY;
         for (int d = 0; d < nbd; d++) {
             nbo[d] = nb_in[d];
@@ -177,7 +179,8 @@ extern "C" int fgc_bin_geometry_f32(const float *d_coords, int64_t n_vert, int32
         return FGC_EINVAL;
     if (!d_coords || !d_geom || !d_ws) return FGC_EINVAL;
     if (ws_bytes < fgc_bin_geometry_workspace_bytes(n_vert)) return FGC_ENOSPACE;
-    if (mode == 0 && (!n_bins_in || !n_bins_given)) return FGC_EINVAL;
+    if (mode < 0 || mode > 2) return FGC_EINVAL;
+    if (mode != 1 && (!n_bins_in || !n_bins_given)) return FGC_EINVAL;
     int nb[FGC_MAX_BIN_DIMS] = {1, 1, 1, 1, 1};
     if (n_bins_in && n_bins_given)
         for (int d = 0; d < n_bin_dims; d++) {
@@ -525,16 +528,19 @@ int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void 
     return FGC_OK;
 }
 
-// bin_boundaries[b] = first sorted position whose key is >= b, for b in [0, n_bins_total]
+// bin_boundaries[b] = first sorted position whose bin is >= b, for b in [0, n_bins_total]: one binary search
+// per bin (long runs of empty bins, e.g. around outliers, cost nothing extra)
 __global__ __launch_bounds__(256) void k_bin_boundaries(const uint32_t *__restrict__ skeys, int n, int shift,
                                                         int n_bins_total, int *__restrict__ bb)
 {
-    int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i > n) return;
-    long long prev = (i > 0) ? (long long)(skeys[i - 1] >> shift) : -1ll;
-    long long cur = (i < n) ? (long long)(skeys[i] >> shift) : (long long)n_bins_total;
-    if (cur > n_bins_total) cur = n_bins_total;
-    for (long long b = prev + 1; b <= cur; b++) bb[b] = i;
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b > n_bins_total) return;
+    int lo = 0, hi = n;
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if ((long long)(skeys[mid] >> shift) < (long long)b) lo = mid + 1; else hi = mid;
+    }
+    bb[b] = lo;
 }
 
 // sorted structure-of-arrays coordinates: sc[d * ldc + i] = coords[order[i]][d]
@@ -565,8 +571,8 @@ int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, int sub_b
 
 int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int shift, int n_bins_total, int *bb, hipStream_t s)
 {
-    hipLaunchKernelGGL(k_bin_boundaries, dim3((unsigned)fgc_cdiv((int64_t)n + 1, 256)), dim3(256), 0, s, skeys,
-                       n, shift, n_bins_total, bb);
+    hipLaunchKernelGGL(k_bin_boundaries, dim3((unsigned)fgc_cdiv((int64_t)n_bins_total + 1, 256)), dim3(256), 0, s,
+                       skeys, n, shift, n_bins_total, bb);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
@@ -598,11 +604,33 @@ __global__ __launch_bounds__(256) void k_chunk_boxes(const float *__restrict__ s
     }
 }
 
-int fgc_launch_chunk_boxes(const float *sc, int n, int D, int ldc, float *box_lo, float *box_hi, hipStream_t s)
+// bounding box of every 64 consecutive chunks (aligned): sbox_lo[d * n_super + g], sbox_hi[d * n_super + g]
+__global__ __launch_bounds__(256) void k_super_boxes(const float *__restrict__ box_lo,
+                                                     const float *__restrict__ box_hi, int D, int n_chunks,
+                                                     int n_super, float *__restrict__ sbox_lo,
+                                                     float *__restrict__ sbox_hi)
+{
+    const int lane = fgc_lane();
+    const int g = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
+    if (g >= n_super) return;
+    const int c = g * 64 + lane;
+    for (int d = 0; d < D; d++) {
+        const float lo = wave_min_f(c < n_chunks ? box_lo[(size_t)d * n_chunks + c] : INFINITY);
+        const float hi = wave_max_f(c < n_chunks ? box_hi[(size_t)d * n_chunks + c] : -INFINITY);
+        if (lane == 0) { sbox_lo[(size_t)d * n_super + g] = lo; sbox_hi[(size_t)d * n_super + g] = hi; }
+    }
+}
+
+int fgc_launch_chunk_boxes(const float *sc, int n, int D, int ldc, float *box_lo, float *box_hi, float *sbox_lo,
+                           float *sbox_hi, hipStream_t s)
 {
     const int n_chunks = ldc / 64;
     hipLaunchKernelGGL(k_chunk_boxes, dim3((unsigned)fgc_cdiv(n_chunks, 4)), dim3(256), 0, s, sc, n, D, ldc,
                        n_chunks, box_lo, box_hi);
+    FGC_LAUNCH_CHECK();
+    const int n_super = (n_chunks + 63) / 64;
+    hipLaunchKernelGGL(k_super_boxes, dim3((unsigned)fgc_cdiv(n_super, 4)), dim3(256), 0, s,
+                       (const float *)box_lo, (const float *)box_hi, D, n_chunks, n_super, sbox_lo, sbox_hi);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }

@@ -8,7 +8,8 @@ int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void 
 int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, int sub_bits, const float *d_geom,
                         const int64_t *d_rs, int n_rs, uint32_t *d_keys, int *d_status, hipStream_t s);
 int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int shift, int n_bins_total, int *bb, hipStream_t s);
-int fgc_launch_chunk_boxes(const float *sc, int n, int D, int ldc, float *box_lo, float *box_hi, hipStream_t s);
+int fgc_launch_chunk_boxes(const float *sc, int n, int D, int ldc, float *box_lo, float *box_hi, float *sbox_lo,
+                           float *sbox_hi, hipStream_t s);
 int fgc_launch_gather_sorted(const float *coords, const uint32_t *order, int n, int D, int ldc, float *sc,
                              const int64_t *direction, unsigned char *sdir, hipStream_t s);
 
@@ -21,6 +22,9 @@ struct KnnArgs {
     const float *box_lo;        // per 64-point chunk bounding boxes [D][n_chunks]
     const float *box_hi;
     int n_chunks;
+    const float *sbox_lo;       // bounding boxes of aligned groups of 64 chunks [D][n_super]
+    const float *sbox_hi;
+    int n_super;
     const uint32_t *order;      // sorted position -> original row
     const int *bb;              // bin boundaries [n_bins_total + 1]
     const float *geom;          // geometry record

@@ -121,6 +121,12 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 #define TM_STOP(acc)
 #endif
     unsigned nchunks = 0, nprunes = 0;
+#ifdef FGC_KNN_COUNTERS
+    unsigned n_cullq = 0, n_app = 0, n_span = 0, n_bis = 0, n_bisx = 0;
+#define CNT(x) x
+#else
+#define CNT(x)
+#endif
     const int slack = max(K >> 2, 4);   // a prune may keep up to K + slack candidates
 
     // ---- shrink query q's pool.  Finds a threshold t with at least K pool entries <= t by bisection
@@ -164,6 +170,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             for (int it = 0; it < iters; it++) {
                 const float mid = 0.5f * (flo + fhi);
                 const int cm = count_le(__float_as_uint(mid));
+                CNT(if (exact) n_bisx++; else n_bis++);
                 if (cm >= K) { fhi = mid; chi = cm; if (cm <= accept) { converged = true; break; } }
                 else flo = mid;
             }
@@ -181,6 +188,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             unsigned lo = 0u;
             while (lo < hi) {
                 const unsigned mid = lo + ((hi - lo) >> 1);
+                CNT(n_bisx++);
                 if (count_le(mid) >= K) hi = mid; else lo = mid + 1u;
             }
             int nless = 0;
@@ -298,10 +306,11 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     for (int i = 0; i < RD; i++)
                         done = done && (need_lo[i] >= cr[i] - (d - 1)) && (need_hi[i] <= cr[i] + (d - 1));
                     if (done) break;
+                    // ring d, clipped to the grid and to the bins the balls can reach
 #pragma unroll
                     for (int i = 0; i < RD; i++) {
-                        lo[i] = max(cr[i] - d, 0);
-                        hi[i] = min(cr[i] + d, rnb[i] - 1);
+                        lo[i] = max(cr[i] - d, need_lo[i]);
+                        hi[i] = min(cr[i] + d, need_hi[i]);
                         ai[i] = lo[i];
                     }
                     ring_open = true; ring_fresh = true; ring_any = false;
@@ -321,14 +330,20 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     }
                 }
                 int cheb = 0, rf = 0;
-                float g2 = gap1(qzn, zlo, zhi, nz);
 #pragma unroll
                 for (int i = 0; i < RD; i++) {
-                    cheb = max(cheb, abs(ai[i] - cr[i]));
+                    if (i < RD - 1) cheb = max(cheb, abs(ai[i] - cr[i]));
                     rf = rf * rnb[i] + ai[i];
-                    g2 += gap1(qb[i], ai[i], ai[i], rnb[i]);
                 }
-                if (cheb != d) continue;
+                if (cheb < d && abs(ai[RD - 1] - cr[RD - 1]) < d) {
+                    // interior of the ring's cube: jump to the far face of the last row dimension (or to the
+                    // end of this line when that face is clipped away)
+                    ai[RD - 1] = (cr[RD - 1] + d <= hi[RD - 1]) ? cr[RD - 1] + d - 1 : hi[RD - 1];
+                    continue;
+                }
+                float g2 = gap1(qzn, zlo, zhi, nz);
+#pragma unroll
+                for (int i = 0; i < RD; i++) g2 += gap1(qb[i], ai[i], ai[i], rnb[i]);
                 ring_any = true;
                 act = gm & fgc_ballot(!(g2 > tau));
                 if (!act) continue;
@@ -341,10 +356,27 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             // ---- one span: sorted positions [j0, j1) against the queries in `act`, chunks sk0..sk1 skipped ----
             const int c0 = j0 >> 6, c1 = (j1 - 1) >> 6;
             const bool cull = (DT > 0) && (c1 - c0 + 1 >= CULL_MIN);
-            for (int cb = c0; cb <= c1; cb += 64) {
+            CNT(n_span++);
+            for (int cb = cull ? (c0 & ~63) : c0; cb <= c1; cb += 64) {
+                unsigned long long actb = act;
+                if (cull) {
+                    // the 64 chunks of this step are one aligned group with a bounding box of its own:
+                    // drop the queries (lane = query) whose ball does not reach it
+                    const int sb = cb >> 6;
+                    float g = fmaxf(fmaxf(a.sbox_lo[sb] - qx[0], qx[0] - a.sbox_hi[sb]), 0.f);
+                    float g2 = g * g;
+#pragma unroll
+                    for (int dd = 1; dd < DR; dd++) {
+                        g = fmaxf(fmaxf(a.sbox_lo[(size_t)dd * a.n_super + sb] - qx[dd],
+                                        qx[dd] - a.sbox_hi[(size_t)dd * a.n_super + sb]), 0.f);
+                        g2 += g * g;
+                    }
+                    actb &= fgc_ballot(!(g2 > tau));
+                    if (!actb) continue;
+                }
                 const int c = cb + lane;
-                const bool cv = (c <= c1) && (c < sk0 || c > sk1);
-                unsigned mymask = cv ? (unsigned)act : 0u;   // queries (bit q) that need chunk c
+                const bool cv = (c >= c0) && (c <= c1) && (c < sk0 || c > sk1);
+                unsigned mymask = cv ? (unsigned)actb : 0u;   // queries (bit q) that need chunk c
                 TM_START();
                 if (cull) {
                     // per-chunk bounding-box test, lane = chunk
@@ -355,7 +387,8 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                         bhi[dd] = cv ? a.box_hi[(size_t)dd * nch + c] : 0.f;
                     }
                     mymask = 0u;
-                    for (unsigned long long m = act; m;) {
+                    for (unsigned long long m = actb; m;) {
+                        CNT(n_cullq++);
                         const int q = __ffsll((long long)m) - 1;
                         m &= m - 1;
                         const float t = fgc_readlane_f(tau, q);
@@ -416,6 +449,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                         unsigned long long pm = fgc_ballot(dsq < t);
                         TM_STOP(tm_eval);
                         if (!pm) continue;
+                        CNT(n_app++);
                         TM_START();
                         // ---- append the passing lanes to query q's pool; when it overflows or runs nearly
                         //      full (tau should stay tight) prune it: first to a tighter threshold, then, if
@@ -532,6 +566,11 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
         atomicAdd(&a.stats[3], tm_cull); atomicAdd(&a.stats[4], tm_eval); atomicAdd(&a.stats[5], tm_pool);
         atomicAdd(&a.stats[6], tm_epi); atomicAdd(&a.stats[7], (unsigned long long)clock64() - tm_total);
 #endif
+#ifdef FGC_KNN_COUNTERS
+        atomicAdd(&a.stats[3], (unsigned long long)n_cullq); atomicAdd(&a.stats[4], (unsigned long long)n_app);
+        atomicAdd(&a.stats[5], (unsigned long long)n_span); atomicAdd(&a.stats[6], (unsigned long long)n_bis);
+        atomicAdd(&a.stats[7], (unsigned long long)n_bisx);
+#endif
         atomicAdd(&a.stats[0], nev);
         atomicAdd(&a.stats[1], (unsigned long long)nchunks);
         atomicAdd(&a.stats[2], (unsigned long long)nprunes);
@@ -567,6 +606,7 @@ template <int NSEG> static int launch_knn_r(const KnnArgs &a, hipStream_t s)
 {
     if (a.nbd <= 2) return launch_knn_d<NSEG, 1>(a, s);
     if (a.nbd == 3) return launch_knn_d<NSEG, 2>(a, s);
+    if (a.nbd == 4) return launch_knn_d<NSEG, 3>(a, s);
     return launch_knn_d<NSEG, 4>(a, s);
 }
 

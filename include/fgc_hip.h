@@ -53,7 +53,10 @@ const char *fgc_error_string(int code);
  * 40-92): global per-dimension minimum, range (+1 where zero, +1e-3), and
  * either the cubic bin width max_d(range_d / n_bins_d) from given n_bins
  * (mode 0) or n_bins_d = int(range_d / bin_width) + 1 from a given width
- * (mode 1).  All in single float32 operations.
+ * (mode 1).  All in single float32 operations.  Mode 2 is mode 0 with the
+ * range padded by a factor 1.001 instead of +1e-3: the grid the kNN search
+ * builds for itself (no counterpart in the reference; the neighbours found do
+ * not depend on the grid).
  *
  *   d_coords     [n_vert, ld_coords] float32, first n_bin_dims columns binned
  *   d_geom       out, float32[FGC_GEOM_FLOATS]: min[5], bin_width, then the

@@ -22,10 +22,20 @@ def _gpu_knn(K, coords, rs, **kw):
 
 
 def _check(oracle, K, coords, rs, threads=8, **kw):
-    gi, gd = _gpu_knn(K, coords, rs, **kw)
+    """GPU result against the checker - with the library's own search grid and, when the caller gives no n_bins,
+    also with the reference's grid (its n_bins heuristic and max_bin_dims)."""
+    from fastgraphcompute_amd import config
+    gi, gd = _gpu_knn(K, coords, rs, **dict(kw))
     okw = {k: (v.cpu().numpy() if torch.is_tensor(v) else v) for k, v in kw.items()}
     oi, od = oracle.binned_select_knn(K, coords, rs, n_threads=threads, **okw)
-    assert_knn_equal(gi, gd, oi, od)
+    assert_knn_equal(gi, gd, oi, od, what="own grid")
+    if kw.get("n_bins") is None:
+        config.auto_grid = False
+        try:
+            ri, rd = _gpu_knn(K, coords, rs, **dict(kw))
+        finally:
+            config.auto_grid = True
+        assert_knn_equal(ri, rd, oi, od, what="reference grid")
     return gi, gd
 
 
