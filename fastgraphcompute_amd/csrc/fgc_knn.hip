@@ -99,7 +99,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     float qx[DR];
     if (DT > 0) {
 #pragma unroll
-        for (int d = 0; d < DR; d++) qx[d] = sc[(size_t)d * ldc + qs];
+        for (int d = 0; d < DR; d++) qx[d] = (d < a.D) ? sc[(size_t)d * ldc + qs] : 0.f;   // padded dimensions: 0
     }
     float qb[RD];  // normalised row-dimension coordinates
 #pragma unroll
@@ -367,9 +367,11 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     float g2 = g * g;
 #pragma unroll
                     for (int dd = 1; dd < DR; dd++) {
-                        g = fmaxf(fmaxf(a.sbox_lo[(size_t)dd * a.n_super + sb] - qx[dd],
-                                        qx[dd] - a.sbox_hi[(size_t)dd * a.n_super + sb]), 0.f);
-                        g2 += g * g;
+                        if (dd < a.D) {
+                            g = fmaxf(fmaxf(a.sbox_lo[(size_t)dd * a.n_super + sb] - qx[dd],
+                                            qx[dd] - a.sbox_hi[(size_t)dd * a.n_super + sb]), 0.f);
+                            g2 += g * g;
+                        }
                     }
                     actb &= fgc_ballot(!(g2 > tau));
                     if (!actb) continue;
@@ -383,8 +385,8 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     float blo[DR], bhi[DR];
 #pragma unroll
                     for (int dd = 0; dd < DR; dd++) {
-                        blo[dd] = cv ? a.box_lo[(size_t)dd * nch + c] : 0.f;
-                        bhi[dd] = cv ? a.box_hi[(size_t)dd * nch + c] : 0.f;
+                        blo[dd] = (cv && dd < a.D) ? a.box_lo[(size_t)dd * nch + c] : 0.f;
+                        bhi[dd] = (cv && dd < a.D) ? a.box_hi[(size_t)dd * nch + c] : 0.f;
                     }
                     mymask = 0u;
                     for (unsigned long long m = actb; m;) {
@@ -417,7 +419,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     float cx[DR];
                     if (DT > 0) {
 #pragma unroll
-                        for (int dd = 0; dd < DR; dd++) cx[dd] = v ? sc[(size_t)dd * ldc + j] : 0.f;
+                        for (int dd = 0; dd < DR; dd++) cx[dd] = (v && dd < a.D) ? sc[(size_t)dd * ldc + j] : 0.f;
                     }
                     bool cand_ok = v;
                     if (a.sdir && v) { unsigned char dd = a.sdir[j]; if (dd == 1 || dd == 2) cand_ok = false; }
@@ -598,8 +600,13 @@ template <int NSEG, int RD> static int launch_knn_d(const KnnArgs &a, hipStream_
     case 6: return launch_knn_t<6, NSEG, RD>(a, s);
     case 7: return launch_knn_t<7, NSEG, RD>(a, s);
     case 8: return launch_knn_t<8, NSEG, RD>(a, s);
-    default: return launch_knn_t<0, NSEG, RD>(a, s);
+    default: break;
     }
+    // more coordinates: padded up to 12 or 16 registers per point (the padding contributes exact zeros),
+    // beyond that read from memory per evaluation
+    if (a.D <= 12) return launch_knn_t<12, NSEG, RD>(a, s);
+    if (a.D <= 16) return launch_knn_t<16, NSEG, RD>(a, s);
+    return launch_knn_t<0, NSEG, RD>(a, s);
 }
 
 template <int NSEG> static int launch_knn_r(const KnnArgs &a, hipStream_t s)

@@ -243,19 +243,49 @@ __global__ __launch_bounds__(256) void k_gravnet_fwd(const int64_t *__restrict__
     const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int64_t i = wave * QPW + sub;
     if (i >= n) return;
-    for (int p = pl; p < P; p += PW) {
+    // The PW lanes of a point first fetch PW neighbour slots together (one coalesced read of the index and
+    // distance rows, one expf per slot instead of one per lane and slot), then every lane walks the slots in
+    // order with the neighbour and its weight broadcast from the lane that fetched them; the gathers of eight
+    // slots are in flight together.
+    const int gbase = sub * PW;
+    for (int p0 = 0; p0 < P; p0 += PW) {
+        const int p = p0 + pl;
+        const bool pv = p < P;
         float s = 0.f, mx = 0.f;
         int am = 0;
-        for (int k = 0; k < K; k++) {
-            const int64_t m = idx[i * K + k];
-            const float w = expf(-10.f * dsq[i * K + k]);
-            const float v = (m == -1 ? 0.f : feat[m * P + p]) * w;
-            s += v;
-            if (k == 0 || v > mx) { mx = v; am = k; }
+        for (int kb = 0; kb < K; kb += PW) {
+            const int kk = kb + pl;
+            int m_l = -1;
+            float w_l = 0.f;
+            if (kk < K) {
+                m_l = (int)idx[i * K + kk];
+                w_l = expf(-10.f * dsq[i * K + kk]);
+            }
+            const int cnt = min(PW, K - kb);
+            for (int j0 = 0; j0 < cnt; j0 += 8) {
+                float f[8], w[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    const int src = gbase + min(j0 + u, PW - 1);
+                    const int m = __shfl(m_l, src, 64);
+                    w[u] = __shfl(w_l, src, 64);
+                    f[u] = (m >= 0 && pv && j0 + u < cnt) ? feat[(int64_t)m * P + p] : 0.f;
+                }
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    if (j0 + u < cnt) {
+                        const float v = f[u] * w[u];
+                        s += v;
+                        if ((kb + j0 + u) == 0 || v > mx) { mx = v; am = kb + j0 + u; }
+                    }
+                }
+            }
         }
-        fmean[i * P + p] = s / (float)K;
-        fmax[i * P + p] = mx;
-        if (argmax) argmax[i * P + p] = am;
+        if (pv) {
+            fmean[i * P + p] = s / (float)K;
+            fmax[i * P + p] = mx;
+            if (argmax) argmax[i * P + p] = am;
+        }
     }
 }
 
@@ -271,24 +301,87 @@ __global__ __launch_bounds__(256) void k_gravnet_bwd(const int64_t *__restrict__
     constexpr int QPW = 64 / PW;
     const int lane = fgc_lane();
     const int sub = lane / PW, pl = lane % PW;
+    const int gbase = sub * PW;
     const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int64_t i = wave * QPW + sub;
     const bool qv = i < n;
     const float invK = 1.0f / (float)K;
-    for (int k = 0; k < K; k++) {
-        const int64_t m = qv ? idx[i * K + k] : -1;
-        const float w = qv ? expf(-10.f * dsq[i * K + k]) : 0.f;
-        float gw = 0.f;  // d loss / d w of this (point, slot)
-        if (m != -1) {
-            for (int p = pl; p < P; p += PW) {
-                const float c = gmean[i * P + p] * invK + (argmax[i * P + p] == k ? gmax[i * P + p] : 0.f);
-                gw += feat[m * P + p] * c;
-                atomicAdd(&gfeat[m * P + p], w * c);
-            }
+    // Slots are fetched PW at a time: lane j of the point's group reads slot kb + j (index, weight).  They are
+    // then visited eight at a time: every lane takes its own feature(s) of the eight neighbours (gathers in
+    // flight together), adds w * c to their feature gradients and keeps one partial dot product per slot; an
+    // exchange across the group's lanes (plain butterflies down to 8 lanes, then halving) leaves the dot
+    // product of slot j0 + (lane & 7) in every lane, and the lane that fetched that slot writes grad_distsq.
+    const bool single = P <= PW;      // one feature per lane: its upstream gradients stay in registers
+    float cm0 = 0.f, gx0 = 0.f;
+    int am0 = -1;
+    if (single && qv && pl < P) {
+        cm0 = gmean[i * P + pl] * invK;
+        gx0 = gmax[i * P + pl];
+        am0 = argmax[i * P + pl];
+    }
+    for (int kb = 0; kb < K; kb += PW) {
+        const int kk = kb + pl;
+        int m_l = -1;
+        float w_l = 0.f;
+        if (qv && kk < K) {
+            m_l = (int)idx[i * K + kk];
+            w_l = expf(-10.f * dsq[i * K + kk]);
         }
+        const int cnt = min(PW, K - kb);
+        for (int j0 = 0; j0 < cnt; j0 += 8) {
+            float vals[8];
+            int m[8];
+            float w[8];
 #pragma unroll
-        for (int o = PW / 2; o > 0; o >>= 1) gw += __shfl_xor(gw, o, 64);
-        if (qv && pl == 0) gdsq[i * K + k] = -10.f * w * gw;
+            for (int u = 0; u < 8; u++) {
+                vals[u] = 0.f;
+                m[u] = __shfl(m_l, gbase + ((j0 + u) & (PW - 1)), 64);
+                w[u] = __shfl(w_l, gbase + ((j0 + u) & (PW - 1)), 64);
+                if (j0 + u >= cnt) m[u] = -1;
+            }
+            for (int p0 = 0; p0 < P; p0 += PW) {
+                const int p = p0 + pl;
+                const bool pv = qv && p < P;
+                float cm = cm0, gx = gx0;
+                int am = am0;
+                if (!single) {
+                    cm = pv ? gmean[i * P + p] * invK : 0.f;
+                    gx = pv ? gmax[i * P + p] : 0.f;
+                    am = pv ? argmax[i * P + p] : -1;
+                }
+                float f[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) f[u] = (m[u] >= 0 && pv) ? feat[(int64_t)m[u] * P + p] : 0.f;
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    if (m[u] >= 0 && pv) {
+                        const float c = cm + (am == kb + j0 + u ? gx : 0.f);
+                        vals[u] += f[u] * c;
+#ifndef FGC_EXPERIMENT_NO_GFEAT_ATOMIC
+                        atomicAdd(&gfeat[(int64_t)m[u] * P + p], w[u] * c);
+#else
+                        vals[u] += w[u] * 1e-30f;
+#endif
+                    }
+                }
+            }
+#pragma unroll
+            for (int sft = PW / 2; sft >= 8; sft >>= 1) {
+#pragma unroll
+                for (int t = 0; t < 8; t++) vals[t] += __shfl_xor(vals[t], sft, 64);
+            }
+#pragma unroll
+            for (int sft = 4; sft >= 1; sft >>= 1) {
+                const bool upper = (pl & sft) != 0;
+#pragma unroll
+                for (int t = 0; t < sft; t++) {
+                    const float send = upper ? vals[t] : vals[t + sft];
+                    const float keep = upper ? vals[t + sft] : vals[t];
+                    vals[t] = keep + __shfl_xor(send, sft, 64);
+                }
+            }
+            if (qv && (pl & ~7) == j0 && kk < K) gdsq[i * K + kk] = -10.f * w_l * vals[0];
+        }
     }
 }
 

@@ -56,7 +56,7 @@ def test_benchmark_shapes_scaled(oracle, name, scale):
     check_knn_properties(gi, gd, w["coords"], w["row_splits"], w["K"])
 
 
-@pytest.mark.parametrize("D", [2, 3, 4, 5, 6, 7, 8, 9, 12])
+@pytest.mark.parametrize("D", [2, 3, 4, 5, 6, 7, 8, 9, 12, 13, 16, 17])
 def test_dimensions(oracle, D):
     rng = np.random.default_rng(40 + D)
     coords = rng.random((3000, D)).astype(np.float32)
