@@ -464,6 +464,48 @@ def _max_same_valued_impl(asso_idx: torch.Tensor, row_splits: torch.Tensor, filt
     return max_per_split, max_per_split.max(), objects_per_split
 
 
+# ------------------------------------------------------------------ brute-force style kNN with a radius limit
+def _select_knn_impl(coords: torch.Tensor, row_splits: torch.Tensor, mask: torch.Tensor, n_neighbours: int,
+                     max_radius: float, mask_mode: int):
+    """select_knn of the reference (select_knn.cpp:60-70): neighbours of the same event within max_radius.
+    mask and mask_mode are accepted and ignored, as in both of the reference's implementations."""
+    _lib.require_device(coords, row_splits)
+    if coords.dim() != 2 or coords.shape[1] == 0:
+        raise ValueError("coords must be [n_vert, n_coords]")
+    K = int(n_neighbours)
+    if K < 1 or K > 256:
+        raise ValueError("select_knn on MI355X supports 1 <= n_neighbours <= 256, got %d" % K)
+    L = _lib.lib()
+    dev = coords.device
+    x = coords.to(torch.float32).contiguous()
+    n, D = x.shape
+    rs_host = row_splits.detach().to("cpu", torch.int64).contiguous()
+    rs_list = rs_host.tolist()
+    n_rs = len(rs_list)
+    if n_rs < 2 or (n > 0 and (rs_list[0] != 0 or rs_list[-1] != n or any(b < a for a, b in zip(rs_list, rs_list[1:])))):
+        raise RuntimeError("row_splits must start at 0, end at the number of points and not decrease")
+    idx = torch.empty((n, K), dtype=torch.int64, device=dev)
+    dist = torch.empty((n, K), dtype=torch.float32, device=dev)
+    if n == 0:
+        return idx, dist
+    if D == 1:                       # the search bins at least two coordinates: add a constant one
+        x = torch.cat([x, torch.zeros_like(x)], dim=1).contiguous()
+        D = 2
+    nbd, nb1 = choose_search_grid(rs_host, D, 3)
+    nb_arr, rs_arr = _lib.host_i64([nb1] * nbd), _lib.host_i64(rs_list)
+    rs_dev = rs_host.to(dev)
+    ws_bytes = L.fgc_binned_select_knn_workspace_bytes(n, D, nbd, nb_arr, n_rs, K)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    status = torch.zeros(4, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(L.fgc_select_knn_f32(_lib.ptr(x), n, D, _lib.ptr(rs_dev), rs_arr, n_rs, K, float(max_radius), nbd,
+                                        nb_arr, _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(status), _lib.ptr(ws),
+                                        ws_bytes, _lib.stream_ptr()))
+    if config.sync_checks and (int(status[0].item()) & _lib.ST_NONFINITE):
+        raise RuntimeError("select_knn: input coordinates contain non-finite values")
+    return idx, dist
+
+
 # ------------------------------------------------------------------ registration
 def _register():
     lib = _define("bin_by_coordinates",
@@ -490,6 +532,12 @@ def _register():
     lib.impl("gravnet_aggregate", _gravnet_aggregate_impl, "Autograd")
     lib.define("select_with_default_f32(Tensor idx, Tensor feat, float default_value) -> Tensor")
     lib.impl("select_with_default_f32", _select_with_default_impl, "Autograd")
+
+    lib = _define("select_knn",
+                  "select_knn(Tensor coords, Tensor row_splits, Tensor mask, int n_neighbours, float max_radius, "
+                  "int mask_mode) -> (Tensor, Tensor)")
+    lib.impl("select_knn", _select_knn_impl, "CUDA")
+    lib.impl("select_knn", _select_knn_impl, "CPU")
 
     lib = _define("oc_helper_cuda",
                   "oc_helper_cuda(Tensor asso_idx, Tensor unique_idx, Tensor unique_rs_asso, Tensor rs, "

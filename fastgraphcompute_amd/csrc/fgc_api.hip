@@ -164,7 +164,8 @@ extern "C" int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert,
                                   (float *)(ws + w.box_hi), (float *)(ws + w.sbox_lo), (float *)(ws + w.sbox_hi), s);
 }
 
-extern "C" int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
+namespace {
+int knn_search(float tau0, int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
                                          int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
                                          int32_t with_direction, int32_t tf_compat, int64_t *d_idx,
                                          float *d_distsq, uint64_t *d_stats, void *d_ws, size_t ws_bytes,
@@ -189,6 +190,7 @@ extern "C" int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const
     a.bb = (const int *)(ws + c.w.bb); a.geom = (const float *)(ws + c.w.geom);
     a.sdir = with_direction ? (const unsigned char *)(ws + c.w.sdir) : nullptr;
     a.n = (int)n_vert; a.D = n_coords; a.nbd = n_bin_dims; a.K = K; a.tf_compat = tf_compat;
+    a.tau0 = tau0;
     a.out_idx = d_idx; a.out_dist = d_distsq; a.stats = (unsigned long long *)d_stats;
     return fgc_launch_knn(a, (hipStream_t)stream);
 }
@@ -207,6 +209,37 @@ extern "C" int fgc_binned_knn_export_order_i32(int64_t n_vert, int32_t n_coords,
     uint32_t *skeys, *order;
     sorted_buffers(c, (char *)const_cast<void *>(d_ws), &skeys, &order);
     return fgc_copy_u32(d_order_out, order, n_vert, (hipStream_t)stream);
+}
+}  // namespace
+
+extern "C" int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
+                                         int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
+                                         int32_t with_direction, int32_t tf_compat, int64_t *d_idx,
+                                         float *d_distsq, uint64_t *d_stats, void *d_ws, size_t ws_bytes,
+                                         void *stream)
+{
+    return knn_search(INFINITY, n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins, with_direction,
+                      tf_compat, d_idx, d_distsq, d_stats, d_ws, ws_bytes, stream);
+}
+
+extern "C" int fgc_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
+                                  const int64_t *d_row_splits, const int64_t *row_splits_host, int32_t n_rs,
+                                  int32_t K, double max_radius, int32_t n_bin_dims, const int64_t *n_bins,
+                                  int64_t *d_idx, float *d_distsq, int32_t *d_status, void *d_ws,
+                                  size_t ws_bytes, void *stream)
+{
+    int rc = fgc_binned_knn_prepare_f32(d_coords, n_vert, n_coords, d_row_splits, row_splits_host, n_rs, K,
+                                        n_bin_dims, n_bins, nullptr, d_status, d_ws, ws_bytes, stream);
+    if (rc) return rc;
+    float tau0 = INFINITY;
+    if (max_radius > 0) {
+        // the reference squares the radius in double, narrows it to float and accepts distsq <= that
+        // (select_knn_cpu.cpp:174-176,110); the search keeps candidates strictly below its bound
+        const float r2 = (float)(max_radius * max_radius);
+        tau0 = nextafterf(r2, INFINITY);
+    }
+    return knn_search(tau0, n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins, 0, 0, d_idx,
+                      d_distsq, nullptr, d_ws, ws_bytes, stream);
 }
 
 extern "C" int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,

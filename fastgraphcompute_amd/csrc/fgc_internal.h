@@ -34,6 +34,7 @@ struct KnnArgs {
     int nbd;                    // binned dimensions
     int K;
     int tf_compat;
+    float tau0;                 // initial bound on the squared neighbour distance (INFINITY: none); exclusive
     int pool_cap;               // candidate pool slots per query (set by fgc_launch_knn)
     int64_t *out_idx;           // [n, K] original order
     float *out_dist;            // [n, K]

@@ -106,7 +106,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     for (int i = 0; i < RD; i++) qb[i] = (i < nbd - 1) ? sc[(size_t)i * ldc + qs] - a.geom[FGC_GEOM_MIN + i] : 0.f;
     const float qzn = sc[(size_t)(nbd - 1) * ldc + qs] - a.geom[FGC_GEOM_MIN + nbd - 1];
     const int row = (int)(a.skeys[qs] >> a.key_shift) / nz;
-    float tau = INFINITY;   // lane q: upper bound of query q's K-th distance
+    float tau = a.tau0;     // lane q: upper bound of query q's K-th distance (starts at the radius bound, if any)
     int cnt = 0;            // lane q: candidates in query q's pool
     bool qactive = isq;
     if (a.sdir && isq) { unsigned char dd = a.sdir[qs]; qactive = !(dd == 0 || dd == 2); }

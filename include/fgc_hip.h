@@ -144,6 +144,23 @@ int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const int64_t *r
                               void *stream);
 
 /* ---------------------------------------------------------------------------
+ * k nearest neighbours inside a radius.  Replaces select_knn_cuda_fn
+ * (select_knn_cuda_kernel.cu:136-212; CPU twin select_knn_cpu.cpp:68-205), the
+ * reference's brute-force search per event: slot 0 the query itself, then its
+ * at most K-1 nearest points of the same event whose squared distance is
+ * <= (float)(max_radius * max_radius), by increasing distance, -1 / 0 padding.
+ * max_radius <= 0 means no limit.  The reference's mask / mask_mode arguments
+ * are read by neither of its implementations and have no counterpart here.
+ * Runs the binned search of fgc_binned_select_knn_f32 with the radius as the
+ * initial bound; workspace and grid arguments as there.
+ */
+int fgc_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
+                       const int64_t *d_row_splits, const int64_t *row_splits_host, int32_t n_rs,
+                       int32_t K, double max_radius, int32_t n_bin_dims, const int64_t *n_bins,
+                       int64_t *d_idx, float *d_distsq, int32_t *d_status, void *d_ws, size_t ws_bytes,
+                       void *stream);
+
+/* ---------------------------------------------------------------------------
  * Replaces index_replacer_cuda_fn (index_replacer_cuda_kernel.cu:30-59):
  * out[i] = in[i] if in[i] < 0 or in[i] >= n_repl, else repl[in[i]].
  */

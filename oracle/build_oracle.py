@@ -21,6 +21,7 @@ REF_TUS = [
     "index_replacer_cpu.cpp",
     "oc_helper_cpu.cpp",
     "oc_helper_helper.cpp",
+    "select_knn_cpu.cpp",
 ]
 
 

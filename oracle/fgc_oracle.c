@@ -399,6 +399,48 @@ int64_t fgc_oracle_oc_calc_m(const int64_t *asso_idx, const int64_t *unique_idx,
     return cut;
 }
 
+/* Brute-force kNN with a radius limit (select_knn_kernel, select_knn_cpu.cpp:68-126, with set_defaults
+ * :49-66 and the radius handling of select_knn_cpu :174-176): per event, slot 0 = the point itself, then up to
+ * K-1 (or event size - 1) other points of the event with distsq <= r2 (any when r2 <= 0): slots fill in index
+ * order, afterwards a candidate strictly closer than the current largest entry replaces it.  Distances are
+ * sequential float sums. */
+void fgc_oracle_select_knn(const float *coord, const int64_t *row_splits, int64_t *idx, float *dist,
+                           int64_t n_vert, int64_t K, int64_t n_coords, int64_t n_rs, double max_radius)
+{
+    if (max_radius > 0) max_radius *= max_radius;
+    const float r2 = (float)max_radius;
+    for (int64_t i = 0; i < n_vert; i++)
+        for (int64_t k = 0; k < K; k++) { idx[i * K + k] = k ? -1 : i; dist[i * K + k] = 0.f; }
+    for (int64_t e = 0; e + 1 < n_rs; e++) {
+        const int64_t lo = row_splits[e], hi = row_splits[e + 1];
+        for (int64_t i = lo; i < hi && i < n_vert; i++) {
+            int64_t maxn = K < hi - lo ? K : hi - lo;
+            int64_t nfilled = 1, maxidx = 0;
+            float maxd = 0.f;
+            for (int64_t j = lo; j < hi; j++) {
+                if (j == i) continue;
+                float d = 0.f;
+                for (int64_t c = 0; c < n_coords; c++) {
+                    float t = coord[i * n_coords + c] - coord[j * n_coords + c];
+                    d += t * t;
+                }
+                if (nfilled < maxn && (r2 <= 0 || r2 >= d)) {
+                    idx[i * K + nfilled] = j; dist[i * K + nfilled] = d;
+                    if (d > maxd) { maxd = d; maxidx = nfilled; }
+                    nfilled++;
+                    continue;
+                }
+                if (d < maxd) {
+                    idx[i * K + maxidx] = j; dist[i * K + maxidx] = d;
+                    maxd = 0.f; maxidx = 0;
+                    for (int64_t n = 1; n < K; n++)
+                        if (dist[i * K + n] > maxd) { maxd = dist[i * K + n]; maxidx = n; }
+                }
+            }
+        }
+    }
+}
+
 int fgc_oracle_max_threads(void)
 {
 #ifdef _OPENMP

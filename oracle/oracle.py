@@ -44,6 +44,9 @@ Pinning status (what fixes each function independently of this restatement):
                                    known answers of tests/test_oc_helper.py:
                                    55-57 and the reference's compiled
                                    oc_helper_helper.cpp (oracle/_ref).
+  select_knn                       the definition (numpy float64 brute force inside the radius), the
+                                   reference's compiled select_knn_cpu (oracle/_ref) slot for slot; the
+                                   reference holds no test or fixture for this op.
   oc_calc_m / oc_helper_matrices   the hand-written expectation of tests/
                                    test_oc_helper.py:80-112, the stored
                                    matrices tests/test_oc_helper_large_M*.npy
@@ -516,3 +519,23 @@ def oc_sort_rows(M, M_not):
     M_not = rows_sorted(np.asarray(M_not)) if M_not is not None else None
     order = np.argsort(M[:, 0], kind="stable") if M.size else np.arange(M.shape[0])
     return M[order], (M_not[order] if M_not is not None else None)
+
+
+# --------------------------------------------------------------------------
+# brute-force kNN with a radius limit
+# --------------------------------------------------------------------------
+def select_knn(K, coords, row_splits, max_radius=-1.0, use_ref=False):
+    """select_knn_cpu, select_knn_cpu.cpp:158-205 (the mask arguments are unused there)."""
+    c = _c(coords, np.float32)
+    rs = _c(row_splits, np.int64)
+    n, D = c.shape
+    idx = np.empty((n, K), dtype=np.int64)
+    dist = np.empty((n, K), dtype=np.float32)
+    args = (_fp(c), _ip(rs), _ip(idx), _fp(dist), ctypes.c_int64(n), ctypes.c_int64(K), ctypes.c_int64(D),
+            ctypes.c_int64(len(rs)), ctypes.c_double(float(max_radius)))
+    if use_ref:
+        if ref_lib().fgc_ref_select_knn(*args):
+            raise RuntimeError("reference select_knn_cpu raised")
+    else:
+        lib().fgc_oracle_select_knn(*args)
+    return idx, dist

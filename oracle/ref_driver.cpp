@@ -3,7 +3,7 @@
 // The functions declared below are defined by the reference's sources
 // (bin_by_coordinates_cpu.cpp:102, binned_select_knn_cpu.cpp:211,
 // binned_select_knn_grad_cpu.cpp:96, index_replacer_cpu.cpp:28,
-// oc_helper_cpu.cpp:118, oc_helper_helper.cpp:30), which
+// oc_helper_cpu.cpp:118, oc_helper_helper.cpp:30, select_knn_cpu.cpp:158), which
 // oracle/build_oracle.py compiles unmodified from the reference checkout.
 // This file only wraps caller memory in tensors and copies results out, so
 // that the checker can call them through ctypes without registering torch
@@ -34,6 +34,11 @@ torch::Tensor index_replacer_cpu_fn(torch::Tensor to_be_replaced,
 std::tuple<torch::Tensor, torch::Tensor> oc_helper_cpu(
     torch::Tensor asso_idx, torch::Tensor unique_idx, torch::Tensor unique_rs_asso, torch::Tensor rs,
     torch::Tensor max_n_unique_over_splits, torch::Tensor max_n_in_splits, bool calc_m_not);
+
+// select_knn_cpu.cpp:158
+std::tuple<torch::Tensor, torch::Tensor> select_knn_cpu(torch::Tensor coords, torch::Tensor row_splits,
+                                                        torch::Tensor mask, int64_t n_neighbours,
+                                                        double max_radius, int64_t mask_mode);
 
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> max_same_valued_entries_per_row_split(
     const torch::Tensor &asso_idx, torch::Tensor row_splits, bool filter_negative);
@@ -133,6 +138,17 @@ int fgc_ref_max_same_valued(const int64_t *asso, const int64_t *rs, int64_t *max
         copy_out<int64_t>(std::get<0>(r), max_per_split);
         global_max[0] = std::get<1>(r).item<int64_t>();
         copy_out<int64_t>(std::get<2>(r), objects_per_split);
+        return 0;
+    } catch (...) { return 1; }
+}
+
+int fgc_ref_select_knn(const float *coord, const int64_t *row_splits, int64_t *idx, float *dist, int64_t n_vert,
+                       int64_t K, int64_t n_coords, int64_t n_rs, double max_radius) {
+    try {
+        auto mask = torch::zeros({n_vert}, torch::kInt64);
+        auto r = select_knn_cpu(f32(coord, {n_vert, n_coords}), i64(row_splits, {n_rs}), mask, K, max_radius, 0);
+        copy_out<int64_t>(std::get<0>(r), idx);
+        copy_out<float>(std::get<1>(r), dist);
         return 0;
     } catch (...) { return 1; }
 }

@@ -1,4 +1,4 @@
-"""Writes tests/golden/ref_cpu_kernels.npz and tests/golden/ref_oc_helper.npz:
+"""Writes tests/golden/ref_cpu_kernels.npz, ref_oc_helper.npz and ref_select_knn.npz:
 outputs of the reference's own CPU kernels (compiled from the reference
 checkout into oracle/_ref by oracle/build_oracle.py) on small seeded inputs.  Run in the build container,
 where the reference checkout exists:
@@ -86,6 +86,23 @@ def make_oc():
     print("wrote", os.path.join(HERE, "ref_oc_helper.npz"))
 
 
+def make_select_knn():
+    out = {}
+    rng = np.random.default_rng(777)
+    for name, n, D, K, rs, radius in (("u3", 1500, 3, 12, [0, 600, 1500], 0.08), ("u3_nolimit", 700, 3, 9, [0, 700], -1.0),
+                                      ("u5", 1200, 5, 20, [0, 5, 5, 1200], 0.35), ("tiny", 6, 2, 8, [0, 6], 0.5)):
+        c = rng.random((n, D)).astype(np.float32)
+        idx, dist = O.select_knn(K, c, np.array(rs), radius, use_ref=True)
+        out[name + "/coords"] = c
+        out[name + "/row_splits"] = np.array(rs, dtype=np.int64)
+        out[name + "/K"] = np.int64(K)
+        out[name + "/max_radius"] = np.float64(radius)
+        out[name + "/idx"] = idx.astype(np.int32)
+        out[name + "/distsq"] = dist
+    np.savez_compressed(os.path.join(HERE, "ref_select_knn.npz"), **out)
+    print("wrote", os.path.join(HERE, "ref_select_knn.npz"))
+
+
 def main():
     if O.ref_lib() is None:
         raise SystemExit("oracle/_ref/libfgc_ref.so missing: run python oracle/build_oracle.py first")
@@ -117,6 +134,7 @@ def main():
     np.savez_compressed(os.path.join(HERE, "ref_cpu_kernels.npz"), **out)
     print("wrote", os.path.join(HERE, "ref_cpu_kernels.npz"))
     make_oc()
+    make_select_knn()
 
 
 if __name__ == "__main__":
