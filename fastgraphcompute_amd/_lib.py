@@ -40,6 +40,8 @@ SIGNATURES = {
                                                      _vp]),
     "fgc_select_knn_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _vp, _i32, _i32, ctypes.c_double, _i32, _vp, _vp, _vp,
                                           _vp, _vp, ctypes.c_size_t, _vp]),
+    "fgc_linear_wgrad_workspace_bytes": (ctypes.c_size_t, [_i64, _i32, _i32]),
+    "fgc_linear_wgrad_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
     "fgc_oc_helper_workspace_bytes": (ctypes.c_size_t, [_i64]),
     "fgc_oc_helper_objects_i64": (ctypes.c_int, [_vp, _i64, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp,
                                                  ctypes.c_size_t, _vp]),

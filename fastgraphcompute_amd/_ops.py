@@ -506,6 +506,60 @@ def _select_knn_impl(coords: torch.Tensor, row_splits: torch.Tensor, mask: torch
     return idx, dist
 
 
+# ------------------------------------------------------------------ dense layer with the library's weight gradient
+def linear_wgrad(grad_out: torch.Tensor, x: torch.Tensor, with_bias: bool = True):
+    """(grad_weight [O, I], grad_bias [O] or None) of y = x W^T + b from grad_out [n, O] and x [n, I]."""
+    _lib.require_device(grad_out, x)
+    L = _lib.lib()
+    g = grad_out.to(torch.float32).contiguous()
+    xx = x.to(torch.float32).contiguous()
+    n, O = g.shape
+    I = xx.shape[1]
+    gw = torch.empty((O, I), dtype=torch.float32, device=g.device)
+    gb = torch.empty(O, dtype=torch.float32, device=g.device) if with_bias else None
+    ws_bytes = L.fgc_linear_wgrad_workspace_bytes(n, O, I)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=g.device)
+    with torch.cuda.device(g.device):
+        _lib.check(L.fgc_linear_wgrad_f32(_lib.ptr(g), _lib.ptr(xx), n, O, I, _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(ws),
+                                          ws_bytes, _lib.stream_ptr()))
+    return gw, gb
+
+
+class _Dense(torch.autograd.Function):
+    """y = x W^T + b.  Forward and input gradient are library GEMMs (tiled over the points, which is what they are
+    good at); the weight gradient, a reduction over the points with a tiny output, is the library's own kernel."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        _lib.require_device(x, weight)
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return torch.nn.functional.linear(x, weight, bias)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight = ctx.saved_tensors
+        gx = gw = gb = None
+        if g is None:
+            return None, None, None
+        g = g.contiguous()
+        if ctx.needs_input_grad[0]:
+            gx = g.matmul(weight)
+        if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
+            x2 = x.reshape(-1, x.shape[-1])
+            g2 = g.reshape(-1, g.shape[-1])
+            if x2.dtype == torch.float32 and g2.dtype == torch.float32:
+                gw, gb = linear_wgrad(g2, x2, ctx.has_bias)
+            else:
+                gw = g2.t().matmul(x2)
+                gb = g2.sum(0) if ctx.has_bias else None
+        return gx, gw, gb
+
+
+def _dense_impl(x, weight, bias):
+    return _Dense.apply(x, weight, bias)
+
+
 # ------------------------------------------------------------------ registration
 def _register():
     lib = _define("bin_by_coordinates",
@@ -530,6 +584,8 @@ def _register():
     lib.impl("binned_select_knn_autograd", _knn_autograd_impl, "Autograd")
     lib.define("gravnet_aggregate(Tensor neighbor_idx, Tensor distsq, Tensor features) -> (Tensor, Tensor)")
     lib.impl("gravnet_aggregate", _gravnet_aggregate_impl, "Autograd")
+    lib.define("dense(Tensor x, Tensor weight, Tensor? bias) -> Tensor")
+    lib.impl("dense", _dense_impl, "Autograd")
     lib.define("select_with_default_f32(Tensor idx, Tensor feat, float default_value) -> Tensor")
     lib.impl("select_with_default_f32", _select_with_default_impl, "Autograd")
 

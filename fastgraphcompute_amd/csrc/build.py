@@ -11,7 +11,7 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["fgc_binning.hip", "fgc_knn.hip", "fgc_ops.hip", "fgc_oc.hip", "fgc_api.hip"]
+SOURCES = ["fgc_binning.hip", "fgc_knn.hip", "fgc_ops.hip", "fgc_oc.hip", "fgc_linear.hip", "fgc_api.hip"]
 OUT = os.path.join(os.path.dirname(HERE), "libfgc_hip.so")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",

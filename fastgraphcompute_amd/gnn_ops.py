@@ -3,7 +3,7 @@ tuple as fastgraphcompute/gnn_ops.py:9-109, so state_dicts interchange; the
 neighbour aggregation (gnn_ops.py:90-102) is one fused HIP kernel per
 direction instead of six tensor ops over a [N, K, P] intermediate.  The module
 is TorchScript-scriptable like the reference's."""
-from typing import Tuple
+from typing import Optional, Tuple
 
 import torch
 
@@ -17,6 +17,13 @@ def gravnet_aggregate(neighbor_idx: torch.Tensor, distsq: torch.Tensor,
     """Mean and max over the K neighbour slots of features[neighbor_idx] * exp(-10 distsq): ([N, P], [N, P]).
     Slots with index -1 contribute 0; the mean always divides by K."""
     return torch.ops.fastgraphcompute_custom_ops.gravnet_aggregate(neighbor_idx, distsq, features)
+
+
+@torch.jit.script
+def dense(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """x W^T + b like torch.nn.functional.linear, with the weight gradient computed by the library's split
+    reduction over the points instead of a tiled GEMM with a tiny output."""
+    return torch.ops.fastgraphcompute_custom_ops.dense(x, weight, bias)
 
 
 class GravNetOp(torch.nn.Module):
@@ -36,10 +43,16 @@ class GravNetOp(torch.nn.Module):
         self.optimization_arguments = optimization_arguments
 
     def forward(self, x: torch.Tensor, row_splits: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-        space = self.space_transformations(x)
-        propagate = self.propagate_transformations(x)
-        neighbor_idx, distsq = binned_select_knn(self.k, space.contiguous(), row_splits)
+        # both projections of x in one product (x is read once, one weight-gradient reduction in the backward)
+        n_space = self.space_transformations.weight.shape[0]
+        w = torch.cat([self.space_transformations.weight, self.propagate_transformations.weight], dim=0)
+        b = torch.cat([self.space_transformations.bias, self.propagate_transformations.bias], dim=0)
+        projected = dense(x, w, b)
+        space = projected[:, :n_space].contiguous()
+        propagate = projected[:, n_space:].contiguous()
+        neighbor_idx, distsq = binned_select_knn(self.k, space, row_splits)
         fmean, fmax = gravnet_aggregate(neighbor_idx, distsq, propagate)
         output = torch.cat([x, fmean, fmax], dim=1)
-        out = self.output_transformations(output)
+        lin = self.output_transformations[0]
+        out = self.output_transformations[1](dense(output, lin.weight, lin.bias))
         return out, neighbor_idx, distsq, space

@@ -224,6 +224,22 @@ int fgc_gravnet_aggregate_bwd_f32(const int64_t *d_idx, const float *d_distsq,
                                   int32_t K, int32_t P, void *stream);
 
 /* ---------------------------------------------------------------------------
+ * Weight and bias gradient of a dense layer y = x W^T + b over n points:
+ *   d_grad_weight [n_out, n_in] = grad_out^T x,  d_grad_bias [n_out] = column sums
+ * of grad_out (NULL to skip).  Replaces the weight-gradient GEMMs that autograd
+ * issues for the three nn.Linear layers of GravNetOp (gnn_ops.py:48-62,79-80,
+ * 105): with n ~ 10^5..10^6 and n_out, n_in <= a few hundred a tiled library
+ * GEMM runs one workgroup per output tile; this splits the points over the
+ * chip (MFMA fp32, fixed summation order).
+ *   d_grad_out [n, n_out], d_input [n, n_in] float32 row-major
+ *   d_ws       fgc_linear_wgrad_workspace_bytes(n, n_out, n_in) bytes
+ */
+size_t fgc_linear_wgrad_workspace_bytes(int64_t n, int32_t n_out, int32_t n_in);
+int fgc_linear_wgrad_f32(const float *d_grad_out, const float *d_input, int64_t n, int32_t n_out,
+                         int32_t n_in, float *d_grad_weight, float *d_grad_bias, void *d_ws,
+                         size_t ws_bytes, void *stream);
+
+/* ---------------------------------------------------------------------------
  * Object-condensation helper matrices.  Two calls with one host read between
  * them (the output shapes depend on the data):
  *
