@@ -90,15 +90,30 @@ __global__ __launch_bounds__(256) void k_linear_wgrad(const float *__restrict__ 
     }
 }
 
-// out[e] = sum over the splits of part[s * count + e], in split order
+// out[e] = sum over the splits of part[s * count + e].  A block owns 64 consecutive outputs; its four wavefronts
+// sum every fourth split (eight loads in flight) and the four sums are added in wavefront order: a fixed order,
+// so the result is reproducible.
 __global__ __launch_bounds__(256) void k_sum_partials(const float *__restrict__ part, int n_splits, int64_t count,
                                                       float *__restrict__ out)
 {
-    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= count) return;
-    float s = 0.f;
-    for (int k = 0; k < n_splits; k++) s += part[(int64_t)k * count + e];
-    out[e] = s;
+    __shared__ float s_sum[4][64];
+    const int lane = fgc_lane(), w = threadIdx.x >> 6;
+    const int64_t e = (int64_t)blockIdx.x * 64 + lane;
+    float acc[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) acc[u] = 0.f;
+    if (e < count) {
+        for (int k0 = w; k0 < n_splits; k0 += 32) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int k = k0 + 4 * u;
+                acc[u] += (k < n_splits) ? part[(int64_t)k * count + e] : 0.f;
+            }
+        }
+    }
+    s_sum[w][lane] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+    __syncthreads();
+    if (w == 0 && e < count) out[e] = (s_sum[0][lane] + s_sum[1][lane]) + (s_sum[2][lane] + s_sum[3][lane]);
 }
 
 struct WgradPlan {
@@ -114,7 +129,7 @@ WgradPlan wgrad_plan(int64_t n, int O, int I)
     p.groups_o = (int)fgc_cdiv(O, 32 * p.tm);
     p.groups_i = (int)fgc_cdiv(I, 32 * WG_TN);
     const int groups = p.groups_o * p.groups_i;
-    int64_t splits = 2048 / groups;                          // about two wavefronts per SIMD over the chip
+    int64_t splits = 1024 / groups;                          // about one wavefront per SIMD over the chip
     const int64_t max_splits = fgc_cdiv(n > 0 ? n : 1, 64);  // at least 64 points per wavefront
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
@@ -162,11 +177,11 @@ extern "C" int fgc_linear_wgrad_f32(const float *d_grad_out, const float *d_inpu
                            p.groups_i, p.n_splits, p.pts_per_split, part_w, part_b);
     FGC_LAUNCH_CHECK();
     const int64_t cw = (int64_t)n_out * n_in;
-    hipLaunchKernelGGL(k_sum_partials, dim3((unsigned)fgc_cdiv(cw, 256)), block, 0, s, (const float *)part_w,
+    hipLaunchKernelGGL(k_sum_partials, dim3((unsigned)fgc_cdiv(cw, 64)), block, 0, s, (const float *)part_w,
                        p.n_splits, cw, d_grad_weight);
     FGC_LAUNCH_CHECK();
     if (d_grad_bias) {
-        hipLaunchKernelGGL(k_sum_partials, dim3((unsigned)fgc_cdiv(n_out, 256)), block, 0, s,
+        hipLaunchKernelGGL(k_sum_partials, dim3((unsigned)fgc_cdiv(n_out, 64)), block, 0, s,
                            (const float *)part_b, p.n_splits, (int64_t)n_out, d_grad_bias);
         FGC_LAUNCH_CHECK();
     }
