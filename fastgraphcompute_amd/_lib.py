@@ -35,6 +35,7 @@ SIGNATURES = {
     "fgc_binned_knn_export_order_i32": (ctypes.c_int, [_i64, _i32, c_i64p, _i32, _i32, _i32, c_i64p, _i32, _vp, _sz,
                                                        _vp, _vp]),
     "fgc_select_with_default_f32": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i32, _i32, _i64, _f32, _vp]),
+    "fgc_select_with_default_b64": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i32, _i32, _i64, ctypes.c_uint64, _vp]),
     "fgc_gravnet_aggregate_fwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp]),
     "fgc_gravnet_aggregate_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32,
                                                      _vp]),

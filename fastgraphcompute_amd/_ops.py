@@ -9,6 +9,7 @@ with `torch.library`; the implementations call libfgc_hip.so through ctypes.
 Two ops have no counterpart in the reference: the fused GravNet aggregation and
 the float32 select_with_default kernel.
 """
+import struct
 from typing import List, Optional, Tuple
 
 import torch
@@ -281,10 +282,19 @@ class _SelectWithDefault(torch.autograd.Function):
         ff = feat.contiguous()
         V, K = ii.shape
         rows, F = ff.shape
-        out = torch.empty((V, K, F), dtype=torch.float32, device=ff.device)
+        out = torch.empty((V, K, F), dtype=ff.dtype, device=ff.device)
         with torch.cuda.device(ff.device):
-            _lib.check(L.fgc_select_with_default_f32(_lib.ptr(ii), _lib.ptr(ff), _lib.ptr(out), V, K, F, rows,
-                                                     float(default_value), _lib.stream_ptr()))
+            if ff.dtype == torch.float32:
+                _lib.check(L.fgc_select_with_default_f32(_lib.ptr(ii), _lib.ptr(ff), _lib.ptr(out), V, K, F, rows,
+                                                         float(default_value), _lib.stream_ptr()))
+            elif ff.dtype in (torch.int64, torch.float64):
+                # 8-byte elements travel as bit patterns; the default is converted as torch.full would do it
+                packed = struct.pack("<q", int(default_value)) if ff.dtype == torch.int64 \
+                    else struct.pack("<d", float(default_value))
+                _lib.check(L.fgc_select_with_default_b64(_lib.ptr(ii), _lib.ptr(ff), _lib.ptr(out), V, K, F, rows,
+                                                         struct.unpack("<Q", packed)[0], _lib.stream_ptr()))
+            else:
+                raise RuntimeError("select_with_default kernel: unsupported feature dtype %s" % ff.dtype)
         ctx.save_for_backward(ii)
         ctx.rows = rows
         return out
@@ -588,6 +598,8 @@ def _register():
     lib.impl("dense", _dense_impl, "Autograd")
     lib.define("select_with_default_f32(Tensor idx, Tensor feat, float default_value) -> Tensor")
     lib.impl("select_with_default_f32", _select_with_default_impl, "Autograd")
+    lib.define("select_with_default_b64(Tensor idx, Tensor feat, float default_value) -> Tensor")
+    lib.impl("select_with_default_b64", _select_with_default_impl, "Autograd")
 
     lib = _define("select_knn",
                   "select_knn(Tensor coords, Tensor row_splits, Tensor mask, int n_neighbours, float max_radius, "

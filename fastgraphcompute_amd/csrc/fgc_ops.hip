@@ -194,33 +194,76 @@ extern "C" int fgc_binned_select_knn_grad_f32(const float *d_grad_distsq, const 
 // ---------------------------------------------------------------------------
 // select_with_default
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void k_select_with_default(const int64_t *__restrict__ idx,
-                                                             const float *__restrict__ feat,
-                                                             float *__restrict__ out, int64_t n_pairs, int F,
-                                                             int64_t n_rows, float dflt)
+// T is the element as a bit pattern (uint32_t for float / int32, uint64_t for int64 / double).
+// Narrow feature rows (F <= 8): one thread per (v, k) pair copies the whole row - one index load, no division.
+template <typename T>
+__global__ __launch_bounds__(256) void k_select_rows(const int64_t *__restrict__ idx, const T *__restrict__ feat,
+                                                     T *__restrict__ out, int64_t n_pairs, int F, int64_t n_rows,
+                                                     T dflt)
 {
-    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    int64_t total = n_pairs * F;
-    if (t >= total) return;
-    int64_t p = t / F;
-    int f = (int)(t - p * F);
-    int64_t m = idx[p];
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= n_pairs) return;
+    const int64_t raw = idx[p];
+    int64_t m = raw;
     if (m < 0) m += n_rows;  // torch advanced indexing wraps negative indices other than the -1 default
-    out[t] = (idx[p] == -1 || m < 0 || m >= n_rows) ? dflt : feat[m * F + f];
+    const bool take = !(raw == -1 || m < 0 || m >= n_rows);
+    T v[8];
+#pragma unroll
+    for (int f = 0; f < 8; f++) v[f] = (take && f < F) ? feat[m * F + f] : dflt;
+#pragma unroll
+    for (int f = 0; f < 8; f++)
+        if (f < F) out[p * F + f] = v[f];
+}
+
+// Wide feature rows: one thread per output element, consecutive lanes on consecutive features.
+template <typename T>
+__global__ __launch_bounds__(256) void k_select_elems(const int64_t *__restrict__ idx, const T *__restrict__ feat,
+                                                      T *__restrict__ out, int64_t n_pairs, int F, int64_t n_rows,
+                                                      T dflt)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_pairs * F) return;
+    int64_t p;
+    if (n_pairs * F < (1ll << 31)) p = (int64_t)((unsigned)t / (unsigned)F); else p = t / F;
+    const int f = (int)(t - p * F);
+    const int64_t raw = idx[p];
+    int64_t m = raw;
+    if (m < 0) m += n_rows;
+    out[t] = (raw == -1 || m < 0 || m >= n_rows) ? dflt : feat[m * F + f];
+}
+
+template <typename T>
+static int select_with_default_launch(const int64_t *d_idx, const T *d_feat, T *d_out, int64_t n_vert, int32_t K,
+                                      int32_t n_feat, int64_t n_feat_rows, T dflt, void *stream)
+{
+    if (n_vert < 0 || K < 0 || n_feat < 0) return FGC_EINVAL;
+    const int64_t pairs = n_vert * K, total = pairs * n_feat;
+    if (total == 0) return FGC_OK;
+    if (n_feat <= 8)
+        hipLaunchKernelGGL((k_select_rows<T>), dim3((unsigned)fgc_cdiv(pairs, 256)), dim3(256), 0,
+                           (hipStream_t)stream, d_idx, d_feat, d_out, pairs, (int)n_feat, n_feat_rows, dflt);
+    else
+        hipLaunchKernelGGL((k_select_elems<T>), dim3((unsigned)fgc_cdiv(total, 256)), dim3(256), 0,
+                           (hipStream_t)stream, d_idx, d_feat, d_out, pairs, (int)n_feat, n_feat_rows, dflt);
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
 }
 
 extern "C" int fgc_select_with_default_f32(const int64_t *d_idx, const float *d_feat, float *d_out,
                                            int64_t n_vert, int32_t K, int32_t n_feat, int64_t n_feat_rows,
                                            float default_value, void *stream)
 {
-    if (n_vert < 0 || K < 0 || n_feat < 0) return FGC_EINVAL;
-    int64_t total = n_vert * K * n_feat;
-    if (total == 0) return FGC_OK;
-    hipLaunchKernelGGL(k_select_with_default, dim3((unsigned)fgc_cdiv(total, 256)), dim3(256), 0,
-                       (hipStream_t)stream, d_idx, d_feat, d_out, n_vert * K, (int)n_feat, n_feat_rows,
-                       default_value);
-    FGC_LAUNCH_CHECK();
-    return FGC_OK;
+    return select_with_default_launch<uint32_t>(d_idx, (const uint32_t *)d_feat, (uint32_t *)d_out, n_vert, K,
+                                                n_feat, n_feat_rows, __builtin_bit_cast(uint32_t, default_value),
+                                                stream);
+}
+
+extern "C" int fgc_select_with_default_b64(const int64_t *d_idx, const void *d_feat, void *d_out, int64_t n_vert,
+                                           int32_t K, int32_t n_feat, int64_t n_feat_rows,
+                                           uint64_t default_bits, void *stream)
+{
+    return select_with_default_launch<uint64_t>(d_idx, (const uint64_t *)d_feat, (uint64_t *)d_out, n_vert, K,
+                                                n_feat, n_feat_rows, default_bits, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -15,6 +15,8 @@ def select_with_default(idx: torch.Tensor, feat: torch.Tensor, default_value: fl
         raise ValueError("select_with_default expects idx [V, K] and feat [V', F]")
     if feat.dtype == torch.float32:
         return torch.ops.fastgraphcompute_custom_ops.select_with_default_f32(idx, feat, default_value)
+    if feat.dtype == torch.int64 or feat.dtype == torch.float64:
+        return torch.ops.fastgraphcompute_custom_ops.select_with_default_b64(idx, feat, default_value)
     # other feature types: the same rule through one gather on a table padded with the default
     rows = feat.shape[0]
     pad = torch.full((1, feat.shape[1]), default_value, dtype=feat.dtype, device=feat.device)

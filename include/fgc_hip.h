@@ -201,6 +201,12 @@ int fgc_binned_knn_export_order_i32(int64_t n_vert, int32_t n_coords, const int6
 int fgc_select_with_default_f32(const int64_t *d_idx, const float *d_feat, float *d_out,
                                 int64_t n_vert, int32_t K, int32_t n_feat, int64_t n_feat_rows,
                                 float default_value, void *stream);
+/* The same for 8-byte elements (int64 or float64 features, as the object-condensation loss selects point
+ * indices and per-event counts, object_condensation.py:148,312); default_bits is the default value's bit
+ * pattern in the element type. */
+int fgc_select_with_default_b64(const int64_t *d_idx, const void *d_feat, void *d_out, int64_t n_vert,
+                                int32_t K, int32_t n_feat, int64_t n_feat_rows, uint64_t default_bits,
+                                void *stream);
 
 /* ---------------------------------------------------------------------------
  * GravNet neighbour aggregation, fused.  Replaces the tensor ops of

@@ -59,6 +59,22 @@ def test_select_with_default(oracle):
     out = select_with_default(torch.from_numpy(idx).cuda(), torch.from_numpy(featl).cuda(), -100)
     assert out.dtype == torch.int64
     np.testing.assert_array_equal(out.cpu().numpy(), oracle.select_with_default(idx, featl, -100))
+    # 8-byte elements with wide rows, float64 with gradient, and other dtypes (generic gather path)
+    for F in (3, 9, 40):
+        featl = rng.integers(-2 ** 40, 2 ** 40, size=(300, F)).astype(np.int64)
+        out = select_with_default(torch.from_numpy(idx).cuda(), torch.from_numpy(featl).cuda(), -1)
+        np.testing.assert_array_equal(out.cpu().numpy(), oracle.select_with_default(idx, featl, -1))
+    featd = torch.from_numpy(rng.standard_normal((300, 5))).cuda().requires_grad_(True)
+    out = select_with_default(torch.from_numpy(idx).cuda(), featd, 0.25)
+    assert out.dtype == torch.float64
+    np.testing.assert_array_equal(out.detach().cpu().numpy(),
+                                  oracle.select_with_default(idx, featd.detach().cpu().numpy(), 0.25))
+    out.sum().backward()
+    counts = np.bincount(idx[idx >= 0], minlength=300).astype(np.float64)
+    np.testing.assert_allclose(featd.grad.cpu().numpy(), np.repeat(counts[:, None], 5, axis=1))
+    feath = torch.from_numpy(rng.standard_normal((300, 4)).astype(np.float16)).cuda()
+    out = select_with_default(torch.from_numpy(idx).cuda(), feath, 2.0)
+    np.testing.assert_array_equal(out.cpu().numpy(), oracle.select_with_default(idx, feath.cpu().numpy(), 2.0))
 
 
 # ---------------------------------------------------------------- kNN gradient
