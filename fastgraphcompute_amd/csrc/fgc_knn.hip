@@ -41,7 +41,7 @@
 #include "fgc_internal.h"
 
 #ifndef QT
-#define QT 8           // queries per wavefront
+#define QT 6           // queries per wavefront (6 x 112 pool slots x 8 B = 5.4 KB of LDS: ~29 wavefronts per CU)
 #endif
 #ifndef POOL_EXTRA
 #define POOL_EXTRA 48  // pool slots beyond K (rounded up to 16); LDS per wavefront = QT * pool slots * 8 B
@@ -57,7 +57,8 @@
 #endif
 
 // wavefronts per block, chosen so that a block's pools fit the 64 KB static LDS limit
-template <int NSEG> struct KnnCfg { static constexpr int WPB = (NSEG <= 2 ? 2 : 1) * (16 / QT); };
+// one wavefront per block: no block-level cooperation is used, and small blocks pack the LDS of a CU best
+template <int NSEG> struct KnnCfg { static constexpr int WPB = 1; };
 
 // DT: coordinates per point held in registers (0 = any number, read from memory)
 // NSEG: ceil(K / 64);  RD: bin-row dimensions (binned dimensions - 1, padded)
@@ -411,7 +412,16 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     }
                 }
                 TM_STOP(tm_cull);
-                for (unsigned long long any = fgc_ballot(mymask != 0u); any;) {
+                // The coordinates of the next surviving chunk are requested before the current one is evaluated
+                // (rows are padded to whole chunks, so a whole chunk can always be read).
+                unsigned long long any = fgc_ballot(mymask != 0u);
+                float nx[DR];
+                if (DT > 0 && any) {
+                    const int jn = ((cb + __ffsll((long long)any) - 1) << 6) + lane;
+#pragma unroll
+                    for (int dd = 0; dd < DR; dd++) nx[dd] = (dd < a.D) ? sc[(size_t)dd * ldc + jn] : 0.f;
+                }
+                while (any) {
                     const int l = __ffsll((long long)any) - 1;
                     any &= any - 1;
                     const unsigned long long cact = (unsigned long long)(unsigned)fgc_readlane_i((int)mymask, l);
@@ -422,7 +432,12 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     float cx[DR];
                     if (DT > 0) {
 #pragma unroll
-                        for (int dd = 0; dd < DR; dd++) cx[dd] = (v && dd < a.D) ? sc[(size_t)dd * ldc + j] : 0.f;
+                        for (int dd = 0; dd < DR; dd++) cx[dd] = nx[dd];
+                        if (any) {
+                            const int jn = ((cb + __ffsll((long long)any) - 1) << 6) + lane;
+#pragma unroll
+                            for (int dd = 0; dd < DR; dd++) nx[dd] = (dd < a.D) ? sc[(size_t)dd * ldc + jn] : 0.f;
+                        }
                     }
                     bool cand_ok = v;
                     if (a.sdir && v) { unsigned char dd = a.sdir[j]; if (dd == 1 || dd == 2) cand_ok = false; }
