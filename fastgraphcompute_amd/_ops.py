@@ -255,6 +255,23 @@ def _knn_autograd_impl(coords, row_splits, K, direction, n_bins, max_bin_dims, t
     return _BinnedKNN.apply(coords, row_splits, K, direction, n_bins, max_bin_dims, torch_compatible_indices)
 
 
+def _knn_sorted_space_impl(coordinates, bin_idx, dim_bin_idx, bin_boundaries, n_bins, bin_width, direction,
+                           tf_compat: bool, use_direction: bool, K: int):
+    """The reference's inner op on already bin-sorted points (binned_select_knn.cpp:82-92): neighbour indices
+    refer to the given (sorted) order.  Events are the groups of prod(n_bins) consecutive bins of
+    bin_boundaries; the search builds its own grid, so bin_idx, dim_bin_idx and bin_width are not needed."""
+    _lib.require_device(coordinates)
+    per_event = int(torch.prod(n_bins.detach().to("cpu", torch.int64)))
+    bb = bin_boundaries.detach().to("cpu", torch.int64)
+    if per_event < 1 or (bb.numel() - 1) % per_event != 0:
+        raise RuntimeError("bin_boundaries must hold prod(n_bins) bins per event plus one entry")
+    row_splits = bb[::per_event].contiguous()
+    d = direction if (use_direction and direction is not None and direction.numel() > 0) else None
+    with torch.no_grad():
+        idx, dist = _BinnedKNN.apply(coordinates, row_splits, int(K), d, None, 3, bool(tf_compat))
+    return idx, dist
+
+
 def _knn_grad_impl(grad_distances, indices, distances, coordinates):
     return knn_grad(grad_distances, indices, coordinates)
 
@@ -587,6 +604,13 @@ def _register():
                   "Tensor coordinates) -> Tensor")
     lib.impl("binned_select_knn_grad", _knn_grad_impl, "CUDA")
     lib.impl("binned_select_knn_grad", _knn_grad_impl, "CPU")
+
+    lib = _define("binned_select_knn",
+                  "binned_select_knn(Tensor coordinates, Tensor bin_idx, Tensor dim_bin_idx, Tensor bin_boundaries, "
+                  "Tensor n_bins, Tensor bin_width, Tensor direction, bool tf_compat, bool use_direction, int K) "
+                  "-> (Tensor, Tensor)")
+    lib.impl("binned_select_knn", _knn_sorted_space_impl, "CUDA")
+    lib.impl("binned_select_knn", _knn_sorted_space_impl, "CPU")
 
     lib = _define("fastgraphcompute_custom_ops",
                   "binned_select_knn_autograd(Tensor coords, Tensor row_splits, int K, Tensor? direction, "

@@ -202,3 +202,22 @@ def test_many_events_with_one_point(oracle):
     rs = np.arange(0, 201, dtype=np.int64)          # 200 events of one point each
     gi, gd = _check(oracle, 4, coords, rs)
     assert (gi[:, 0] == np.arange(200)).all() and (gi[:, 1:] == -1).all()
+
+
+def test_sorted_space_op(oracle):
+    """torch.ops.binned_select_knn.binned_select_knn, the reference's inner op on bin-sorted input
+    (binned_select_knn.cpp:82-92): indices refer to the sorted order."""
+    import fastgraphcompute_amd  # noqa: F401  (registers the ops)
+    rng = np.random.default_rng(77)
+    coords = rng.random((4000, 3)).astype(np.float32)
+    rs = np.array([0, 1500, 4000])
+    direction = rng.integers(0, 3, 4000)
+    s = oracle.sorted_space(coords, rs, 12, direction=direction)
+    t = lambda a: torch.as_tensor(np.ascontiguousarray(a), device="cuda")
+    for use_dir in (False, True):
+        oi, od, _, _ = oracle.knn_sorted(s["scoords"], s["sbin"], s["sdbin"], s["bin_boundaries"], s["n_bins"],
+                                         s["bin_width"], 12, sdirection=s["sdirection"] if use_dir else None)
+        gi, gd = torch.ops.binned_select_knn.binned_select_knn(
+            t(s["scoords"]), t(s["sbin"]), t(s["sdbin"]), t(s["bin_boundaries"]), t(s["n_bins"]), t(s["bin_width"]),
+            t(s["sdirection"]), False, use_dir, 12)
+        assert_knn_equal(gi.cpu().numpy(), gd.cpu().numpy(), oi, od, what="direction %s" % use_dir)
