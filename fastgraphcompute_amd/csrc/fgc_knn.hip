@@ -46,14 +46,17 @@
 #ifndef POOL_EXTRA
 #define POOL_EXTRA 48  // pool slots beyond K (rounded up to 16); LDS per wavefront = QT * pool slots * 8 B
 #endif
+#ifndef POOL_EXTRA_SMALL_K
+#define POOL_EXTRA_SMALL_K 64
+#endif
 #ifndef PRUNE_MARGIN
-#define PRUNE_MARGIN 8 // a pool is pruned when fewer than this many slots are free
+#define PRUNE_MARGIN 24 // a pool is pruned when fewer than this many slots are free
 #endif
 #ifndef SEED_W
 #define SEED_W 1     // seed chunks on either side of the wavefront's own chunk, per 64 neighbours asked for
 #endif
 #ifndef CULL_MIN
-#define CULL_MIN 3     // spans of at least this many chunks get the per-chunk box test
+#define CULL_MIN 5     // spans of at least this many chunks get the per-chunk box test
 #endif
 
 // wavefronts per block, chosen so that a block's pools fit the 64 KB static LDS limit
@@ -131,7 +134,10 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 #else
 #define CNT(x)
 #endif
-    const int slack = max(K >> 2, 4);   // a prune may keep up to K + slack candidates
+#ifndef SLACK_SHIFT
+#define SLACK_SHIFT 3
+#endif
+    const int slack = max(K >> SLACK_SHIFT, 4);   // a prune may keep up to K + slack candidates
 
     // ---- shrink query q's pool.  Finds a threshold t with at least K pool entries <= t by bisection
     //      (counts via wave ballots, the pool held one slot per lane and segment), keeps the entries
@@ -641,7 +647,9 @@ int fgc_launch_knn(const KnnArgs &a_in, hipStream_t s)
     if (a.n <= 0) return FGC_OK;
     if (a.K < 1 || a.K > FGC_MAX_K || a.D < 1 || a.nbd < 1 || a.nbd > FGC_MAX_BIN_DIMS || a.nbd > a.D)
         return FGC_EINVAL;
-    a.pool_cap = ((a.K + POOL_EXTRA + 15) / 16) * 16;   // <= 64 * (ceil(K / 64) + 1)
+    // K kept + room for new candidates: a whole chunk for K <= 64, where LDS is not yet what limits the number
+    // of resident wavefronts, less beyond; always <= 64 * (ceil(K / 64) + 1)
+    a.pool_cap = ((a.K + (a.K <= 64 ? POOL_EXTRA_SMALL_K : POOL_EXTRA) + 15) / 16) * 16;
     if (a.K <= 64) return launch_knn_r<1>(a, s);
     if (a.K <= 128) return launch_knn_r<2>(a, s);
     return launch_knn_r<4>(a, s);
