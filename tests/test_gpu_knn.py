@@ -221,3 +221,49 @@ def test_sorted_space_op(oracle):
             t(s["scoords"]), t(s["sbin"]), t(s["sdbin"]), t(s["bin_boundaries"]), t(s["n_bins"]), t(s["bin_width"]),
             t(s["sdirection"]), False, use_dir, 12)
         assert_knn_equal(gi.cpu().numpy(), gd.cpu().numpy(), oi, od, what="direction %s" % use_dir)
+
+
+def _adversarial(name, n, rng):
+    if name == "line":                       # a 1-D manifold in 3-D
+        t = rng.random(n)
+        return np.stack([t, 2 * t + 0.5, -t], axis=1)
+    if name == "plane":
+        c = rng.random((n, 3))
+        c[:, 2] = 0.25 * c[:, 0] - c[:, 1]
+        return c
+    if name == "offset":                     # a small cloud far from the origin: few mantissa bits left
+        return 1.0e6 + rng.random((n, 3))
+    if name == "tiny":
+        return rng.random((n, 3)) * 1e-18
+    if name == "huge":
+        return (rng.random((n, 3)) - 0.5) * 1e15
+    if name == "lattice":                    # massive ties
+        return rng.integers(0, 7, size=(n, 3)).astype(np.float64)
+    if name == "cauchy":                     # heavy tails: a dense core and far outliers
+        return rng.standard_cauchy((n, 3))
+    if name == "constant_dim":
+        c = rng.random((n, 4))
+        c[:, 1] = 3.5
+        return c
+    if name == "two_scales":                 # one tight blob next to a wide one
+        c = rng.standard_normal((n, 3))
+        c[: n // 2] *= 1e-4
+        return c
+    if name == "shell":                      # points on a sphere: every query's ball is mostly empty space
+        v = rng.standard_normal((n, 3))
+        return v / np.linalg.norm(v, axis=1, keepdims=True)
+    raise ValueError(name)
+
+
+@pytest.mark.parametrize("name", ["line", "plane", "offset", "tiny", "huge", "lattice", "cauchy", "constant_dim",
+                                  "two_scales", "shell"])
+def test_adversarial_distributions(oracle, name):
+    """Distributions that stress the bin / bounding-box filters: the result must still be the exact kNN."""
+    rng = np.random.default_rng(sum(map(ord, name)))
+    coords = _adversarial(name, 6000, rng).astype(np.float32)
+    rs = [0, 2500, 6000]
+    for K in (8, 70):
+        bi, bd = oracle.knn_brute(K, coords, np.array(rs))
+        for n_bins in (None, 11, 29):        # the library's own coarse grid, and fine grids with many rings
+            gi, gd = _gpu_knn(K, coords, rs, n_bins=None if n_bins is None else torch.tensor(n_bins))
+            assert_knn_equal(gi, gd, bi, bd, what="%s K=%d n_bins=%s" % (name, K, n_bins))
