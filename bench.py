@@ -105,7 +105,7 @@ def main():
     ws_bytes = L.fgc_binned_select_knn_workspace_bytes(n, D, nbd, nb_arr, n_rs, K)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     status = torch.zeros(4, dtype=torch.int32, device=dev)
-    stats = torch.zeros(4, dtype=torch.int64, device=dev)
+    stats = torch.zeros(8, dtype=torch.int64, device=dev)
     idx = torch.empty((n, K), dtype=torch.int64, device=dev)
     dist = torch.empty((n, K), dtype=torch.float32, device=dev)
     st = _lib.stream_ptr()
@@ -163,7 +163,7 @@ def main():
         "forward_queries_per_s": round(n / ((t_prep + t_knn) * 1e-3), 1),
         "stages_ms": {"bin_sort_gather": round(t_prep, 4), "knn_search": round(t_knn, 4),
                       "gradient": round(t_grad, 4)},
-        "search_counters": {"distance_evaluations": c_eval, "candidate_chunks": chunks, "insertions": inserts},
+        "search_counters": {"distance_evaluations": c_eval, "candidate_chunks": chunks, "pool_prunes": inserts},
         "roofline": roofline,
     }
 

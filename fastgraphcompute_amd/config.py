@@ -6,7 +6,7 @@
 sync_checks = True
 
 # Accumulate the kNN kernel's counters (distance evaluations, candidate chunks,
-# list insertions) into binned_select_knn.last_stats; used by the benchmark.
+# pool prunes) into binned_select_knn.last_stats; used by the benchmark.
 collect_stats = False
 
 # When binned_select_knn is called without n_bins, size the search grid for this library's search (coarse bins

@@ -119,14 +119,6 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     if (a.sdir && isq) { unsigned char dd = a.sdir[qs]; qactive = !(dd == 0 || dd == 2); }
 
     unsigned long long nev = 0;
-#ifdef FGC_KNN_TIMERS
-    unsigned long long tm_cull = 0, tm_eval = 0, tm_pool = 0, tm_epi = 0, tm_total = clock64(), tm0;
-#define TM_START() tm0 = clock64()
-#define TM_STOP(acc) acc += clock64() - tm0
-#else
-#define TM_START()
-#define TM_STOP(acc)
-#endif
     unsigned nchunks = 0, nprunes = 0;
 #ifdef FGC_KNN_COUNTERS
     unsigned n_cullq = 0, n_app = 0, n_span = 0, n_bis = 0, n_bisx = 0;
@@ -389,7 +381,6 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                 const int c = cb + lane;
                 const bool cv = (c >= c0) && (c <= c1) && (c < sk0 || c > sk1);
                 unsigned mymask = cv ? (unsigned)actb : 0u;   // queries (bit q) that need chunk c
-                TM_START();
                 if (cull) {
                     // per-chunk bounding-box test, lane = chunk
                     float blo[DR], bhi[DR];
@@ -417,7 +408,6 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                         if (cv && !(g2 > t)) mymask |= 1u << q;
                     }
                 }
-                TM_STOP(tm_cull);
                 // The coordinates of the next surviving chunk are requested before the current one is evaluated
                 // (rows are padded to whole chunks, so a whole chunk can always be read).
                 unsigned long long any = fgc_ballot(mymask != 0u);
@@ -451,7 +441,6 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     nev += (unsigned long long)__popcll(cact) * (unsigned)(min(j1, base + 64) - max(j0, base));
                     nchunks++;
                     for (unsigned long long m = cact; m;) {
-                        TM_START();
                         const int q = __ffsll((long long)m) - 1;
                         m &= m - 1;
                         const float t = fgc_readlane_f(tau, q);
@@ -473,10 +462,8 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                             }
                         }
                         unsigned long long pm = fgc_ballot(dsq < t);
-                        TM_STOP(tm_eval);
                         if (!pm) continue;
                         CNT(n_app++);
-                        TM_START();
                         // ---- append the passing lanes to query q's pool; when it overflows or runs nearly
                         //      full (tau should stay tight) prune it: first to a tighter threshold, then, if
                         //      lanes are still waiting, down to exactly K ----
@@ -501,7 +488,6 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                             pm = fgc_ballot(((pm >> lane) & 1ull) && rnk >= room && dsq < fgc_readlane_f(tau, q));
                             if (!pm) break;
                         }
-                        TM_STOP(tm_pool);
                     }
                 }
             }
@@ -510,13 +496,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 
     // ---- per query: cut the pool to exactly K, sort by distance, write the row at the query's
     //      original position (slot 0 = the query itself) ----
-    TM_START();
-#ifdef FGC_EXPERIMENT_NO_EPILOGUE
-    if (lane < nq) a.out_dist[(long long)a.order[qbeg + lane] * K] = tau;
-    for (int q = 0; q < 0; q++) {
-#else
     for (int q = 0; q < nq; q++) {
-#endif
         const int self = qbeg + q;
         const long long orig_q = (long long)a.order[self];
         prune(q, true);
@@ -586,12 +566,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             }
         }
     }
-    TM_STOP(tm_epi);
     if (a.stats && lane == 0) {
-#ifdef FGC_KNN_TIMERS
-        atomicAdd(&a.stats[3], tm_cull); atomicAdd(&a.stats[4], tm_eval); atomicAdd(&a.stats[5], tm_pool);
-        atomicAdd(&a.stats[6], tm_epi); atomicAdd(&a.stats[7], (unsigned long long)clock64() - tm_total);
-#endif
 #ifdef FGC_KNN_COUNTERS
         atomicAdd(&a.stats[3], (unsigned long long)n_cullq); atomicAdd(&a.stats[4], (unsigned long long)n_app);
         atomicAdd(&a.stats[5], (unsigned long long)n_span); atomicAdd(&a.stats[6], (unsigned long long)n_bis);

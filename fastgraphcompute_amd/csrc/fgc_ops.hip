@@ -400,11 +400,7 @@ __global__ __launch_bounds__(256) void k_gravnet_bwd(const int64_t *__restrict__
                     if (m[u] >= 0 && pv) {
                         const float c = cm + (am == kb + j0 + u ? gx : 0.f);
                         vals[u] += f[u] * c;
-#ifndef FGC_EXPERIMENT_NO_GFEAT_ATOMIC
                         atomicAdd(&gfeat[(int64_t)m[u] * P + p], w[u] * c);
-#else
-                        vals[u] += w[u] * 1e-30f;
-#endif
                     }
                 }
             }

@@ -112,9 +112,10 @@ int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t ld_coords,
  *                 -1 (or the query's index if tf_compat) where the event has
  *                 fewer than K points
  *   d_distsq      out float32 [n_vert, K], 0 for slot 0 and for padding
- *   d_stats       optional uint64[4] device counters, accumulated: [0] distance
- *                 evaluations, [1] candidate chunks visited, [2] pool prunes;
- *                 NULL to skip
+ *   d_stats       optional uint64[8] device counters, accumulated: [0] distance
+ *                 evaluations, [1] candidate chunks visited, [2] pool prunes
+ *                 ([3..7] only in debug builds with -DFGC_KNN_COUNTERS: box
+ *                 tests, appends, spans, bisection steps); NULL to skip
  */
 size_t fgc_binned_select_knn_workspace_bytes(int64_t n_vert, int32_t n_coords,
                                              int32_t n_bin_dims, const int64_t *n_bins,
