@@ -160,6 +160,20 @@ def knn_grad(grad_distsq: torch.Tensor, idx: torch.Tensor, coords: torch.Tensor,
     return out
 
 
+_PINNED = {}
+
+
+def _pinned_status(dev: torch.device) -> torch.Tensor:
+    """One pinned int32[4] per device for the asynchronous read-back of the status word (each use ends with a
+    wait on its own event, so the buffer is free again when the next call starts)."""
+    key = dev.index if dev.index is not None else torch.cuda.current_device()
+    buf = _PINNED.get(key)
+    if buf is None:
+        buf = torch.empty(4, dtype=torch.int32, pin_memory=True)
+        _PINNED[key] = buf
+    return buf
+
+
 class _BinnedKNN(torch.autograd.Function):
     @staticmethod
     def forward(ctx, coords, row_splits, K, direction, n_bins, max_bin_dims, tf_compat):
@@ -215,18 +229,30 @@ class _BinnedKNN(torch.autograd.Function):
                 dirt = direction.to(device=dev, dtype=torch.int64).contiguous()
             with torch.cuda.device(dev):
                 st = _lib.stream_ptr()
-                _lib.check(L.fgc_binned_select_knn_f32(
+                # prepare and search are enqueued separately so that the input checks (status word, written by
+                # the prepare stage) can be read back while the search is already queued behind them: the host
+                # then waits for the short prepare stage only and the device never runs dry
+                _lib.check(L.fgc_binned_knn_prepare_f32(
                     _lib.ptr(coords), n, D, _lib.ptr(rs_dev), rs_arr, n_rs, K, nbd, nb_arr, _lib.ptr(dirt),
-                    1 if tf_compat else 0, _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(status), _lib.ptr(stats),
-                    _lib.ptr(ws), ws_bytes, st))
+                    _lib.ptr(status), _lib.ptr(ws), ws_bytes, st))
+                checked = None
+                if config.sync_checks:
+                    status_host = _pinned_status(dev)
+                    status_host.copy_(status, non_blocking=True)
+                    checked = torch.cuda.Event()
+                    checked.record()
+                _lib.check(L.fgc_binned_knn_search_f32(
+                    n, D, rs_arr, n_rs, K, nbd, nb_arr, 1 if dirt is not None else 0, 1 if tf_compat else 0,
+                    _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(stats), _lib.ptr(ws), ws_bytes, st))
                 if ctx.needs_input_grad[0]:
                     # the backward processes queries in the forward's bin-sorted order
                     order = torch.empty(n, dtype=torch.int32, device=dev)
                     _lib.check(L.fgc_binned_knn_export_order_i32(n, D, rs_arr, n_rs, K, nbd, nb_arr,
                                                                  1 if dirt is not None else 0, _lib.ptr(ws),
                                                                  ws_bytes, _lib.ptr(order), st))
-            if config.sync_checks:
-                flags = int(status[0].item())
+            if checked is not None:
+                checked.synchronize()
+                flags = int(status_host[0])
                 if flags & _lib.ST_NONFINITE:
                     raise RuntimeError("BinByCoordinates: input coordinates contain non-finite values")
                 if flags & _lib.ST_BAD_RANGE:
