@@ -46,7 +46,7 @@ def main():
     from fastgraphcompute_amd import _lib, config, workloads
     from fastgraphcompute_amd.extensions.binned_select_knn import (binned_select_knn_grad,
                                                                    calculate_optimal_bins)
-    from fastgraphcompute_amd._ops import choose_search_grid
+    from fastgraphcompute_amd._ops import choose_search_grid, knn_grad_sorted
 
     if not torch.cuda.is_available():
         print("bench.py: no HIP device visible", file=sys.stderr)
@@ -108,6 +108,7 @@ def main():
     stats = torch.zeros(8, dtype=torch.int64, device=dev)
     idx = torch.empty((n, K), dtype=torch.int64, device=dev)
     dist = torch.empty((n, K), dtype=torch.float32, device=dev)
+    nbr_sorted = torch.empty((n, K), dtype=torch.int32, device=dev)   # as the autograd path requests it
     st = _lib.stream_ptr()
 
     def prepare():
@@ -116,6 +117,7 @@ def main():
 
     def search(with_stats):
         _lib.check(L.fgc_binned_knn_search_f32(n, D, rs_arr, n_rs, K, nbd, nb_arr, 0, 0, _lib.ptr(idx), _lib.ptr(dist),
+                                               _lib.ptr(nbr_sorted),
                                                _lib.ptr(stats) if with_stats else None, _lib.ptr(ws), ws_bytes, st))
 
     def timed(fn, reps):
@@ -139,7 +141,7 @@ def main():
     order = torch.empty(n, dtype=torch.int32, device=dev)
     _lib.check(L.fgc_binned_knn_export_order_i32(n, D, rs_arr, n_rs, K, nbd, nb_arr, 0, _lib.ptr(ws), ws_bytes,
                                                  _lib.ptr(order), st))
-    t_grad = float(np.mean(timed(lambda: binned_select_knn_grad(grad_d, idx, coords, order), reps)))
+    t_grad = float(np.mean(timed(lambda: knn_grad_sorted(grad_d, nbr_sorted, coords, order), reps)))
 
     # algorithmic bytes of one search launch: every distance evaluation reads one
     # D-float candidate, every query is read once, every (idx, distsq) slot written once

@@ -174,6 +174,27 @@ def _pinned_status(dev: torch.device) -> torch.Tensor:
     return buf
 
 
+def knn_grad_sorted(grad_distsq: torch.Tensor, nbr_sorted: torch.Tensor, coords: torch.Tensor,
+                    order: torch.Tensor) -> torch.Tensor:
+    """d(loss)/d(coords) from d(loss)/d(distsq) with the neighbour rows and permutation of the forward's sorted
+    order (what binned_select_knn keeps for its backward)."""
+    _lib.require_device(grad_distsq, nbr_sorted, coords, order)
+    L = _lib.lib()
+    g = grad_distsq.to(torch.float32).contiguous()
+    x = coords.to(torch.float32).contiguous()
+    n, D = x.shape
+    K = nbr_sorted.shape[1]
+    out = torch.empty((n, D), dtype=torch.float32, device=x.device)
+    status = torch.zeros(4, dtype=torch.int32, device=x.device)
+    ws_bytes = L.fgc_binned_select_knn_grad_sorted_workspace_bytes(n, D)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(L.fgc_binned_select_knn_grad_sorted_f32(_lib.ptr(g), _lib.ptr(nbr_sorted), _lib.ptr(x),
+                                                           _lib.ptr(order), _lib.ptr(out), n, K, D, _lib.ptr(status),
+                                                           _lib.ptr(ws), ws_bytes, _lib.stream_ptr()))
+    return out
+
+
 class _BinnedKNN(torch.autograd.Function):
     @staticmethod
     def forward(ctx, coords, row_splits, K, direction, n_bins, max_bin_dims, tf_compat):
@@ -217,6 +238,7 @@ class _BinnedKNN(torch.autograd.Function):
         idx = torch.empty((n, K), dtype=torch.int64, device=dev)
         dist = torch.empty((n, K), dtype=torch.float32, device=dev)
         order = torch.empty(0, dtype=torch.int32, device=dev)
+        nbr_sorted = None
         if n > 0:
             nb_arr = _lib.host_i64(nb)
             rs_arr = _lib.host_i64(rs_list)
@@ -241,11 +263,14 @@ class _BinnedKNN(torch.autograd.Function):
                     status_host.copy_(status, non_blocking=True)
                     checked = torch.cuda.Event()
                     checked.record()
+                if ctx.needs_input_grad[0]:
+                    # the backward works in the search's sorted order: it gets the neighbour rows in that order
+                    # (int32) and the permutation
+                    nbr_sorted = torch.empty((n, K), dtype=torch.int32, device=dev)
                 _lib.check(L.fgc_binned_knn_search_f32(
                     n, D, rs_arr, n_rs, K, nbd, nb_arr, 1 if dirt is not None else 0, 1 if tf_compat else 0,
-                    _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(stats), _lib.ptr(ws), ws_bytes, st))
+                    _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(nbr_sorted), _lib.ptr(stats), _lib.ptr(ws), ws_bytes, st))
                 if ctx.needs_input_grad[0]:
-                    # the backward processes queries in the forward's bin-sorted order
                     order = torch.empty(n, dtype=torch.int32, device=dev)
                     _lib.check(L.fgc_binned_knn_export_order_i32(n, D, rs_arr, n_rs, K, nbd, nb_arr,
                                                                  1 if dirt is not None else 0, _lib.ptr(ws),
@@ -261,19 +286,21 @@ class _BinnedKNN(torch.autograd.Function):
                 s = stats.tolist()
                 last_stats.update(distance_evaluations=s[0], candidate_chunks=s[1], pool_prunes=s[2],
                                   n_bins=nb, n_vert=n, K=K, n_coords=D)
-        ctx.save_for_backward(idx, coords, order)
+        if nbr_sorted is None:
+            nbr_sorted = torch.empty((0, K), dtype=torch.int32, device=dev)
+        ctx.save_for_backward(nbr_sorted, coords, order)
         ctx.mark_non_differentiable(idx)
         ctx.set_materialize_grads(False)   # no zero tensors for unused output gradients
         return idx, dist
 
     @staticmethod
     def backward(ctx, _grad_idx, grad_dist):
-        idx, coords, order = ctx.saved_tensors
+        nbr_sorted, coords, order = ctx.saved_tensors
         if not ctx.needs_input_grad[0]:
             return None, None, None, None, None, None, None
-        if grad_dist is None:
+        if grad_dist is None or coords.shape[0] == 0:
             return torch.zeros_like(coords), None, None, None, None, None, None
-        g = knn_grad(grad_dist, idx, coords, order if order.numel() else None)
+        g = knn_grad_sorted(grad_dist, nbr_sorted, coords, order)
         return g, None, None, None, None, None, None
 
 

@@ -165,7 +165,7 @@ extern "C" int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert,
 }
 
 namespace {
-int knn_search(float tau0, int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
+int knn_search(float tau0, int32_t *d_nbr_sorted, int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
                                          int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
                                          int32_t with_direction, int32_t tf_compat, int64_t *d_idx,
                                          float *d_distsq, uint64_t *d_stats, void *d_ws, size_t ws_bytes,
@@ -191,6 +191,7 @@ int knn_search(float tau0, int64_t n_vert, int32_t n_coords, const int64_t *row_
     a.sdir = with_direction ? (const unsigned char *)(ws + c.w.sdir) : nullptr;
     a.n = (int)n_vert; a.D = n_coords; a.nbd = n_bin_dims; a.K = K; a.tf_compat = tf_compat;
     a.tau0 = tau0;
+    a.out_sorted = d_nbr_sorted;
     a.out_idx = d_idx; a.out_dist = d_distsq; a.stats = (unsigned long long *)d_stats;
     return fgc_launch_knn(a, (hipStream_t)stream);
 }
@@ -215,10 +216,10 @@ extern "C" int fgc_binned_knn_export_order_i32(int64_t n_vert, int32_t n_coords,
 extern "C" int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
                                          int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
                                          int32_t with_direction, int32_t tf_compat, int64_t *d_idx,
-                                         float *d_distsq, uint64_t *d_stats, void *d_ws, size_t ws_bytes,
-                                         void *stream)
+                                         float *d_distsq, int32_t *d_nbr_sorted, uint64_t *d_stats, void *d_ws,
+                                         size_t ws_bytes, void *stream)
 {
-    return knn_search(INFINITY, n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins, with_direction,
+    return knn_search(INFINITY, d_nbr_sorted, n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins, with_direction,
                       tf_compat, d_idx, d_distsq, d_stats, d_ws, ws_bytes, stream);
 }
 
@@ -238,7 +239,7 @@ extern "C" int fgc_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t
         const float r2 = (float)(max_radius * max_radius);
         tau0 = nextafterf(r2, INFINITY);
     }
-    return knn_search(tau0, n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins, 0, 0, d_idx,
+    return knn_search(tau0, nullptr, n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins, 0, 0, d_idx,
                       d_distsq, nullptr, d_ws, ws_bytes, stream);
 }
 
@@ -253,6 +254,6 @@ extern "C" int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, 
                                         n_bin_dims, n_bins, d_direction, d_status, d_ws, ws_bytes, stream);
     if (rc) return rc;
     return fgc_binned_knn_search_f32(n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins,
-                                     d_direction != nullptr, tf_compat, d_idx, d_distsq, d_stats, d_ws, ws_bytes,
-                                     stream);
+                                     d_direction != nullptr, tf_compat, d_idx, d_distsq, nullptr, d_stats, d_ws,
+                                     ws_bytes, stream);
 }

@@ -38,6 +38,8 @@ struct KnnArgs {
     int pool_cap;               // candidate pool slots per query (set by fgc_launch_knn)
     int64_t *out_idx;           // [n, K] original order
     float *out_dist;            // [n, K]
+    int *out_sorted;            // optional [n, K]: the same rows in sorted space (row = sorted position of the
+                                // query, entries = sorted positions), for the gradient kernel
     unsigned long long *stats;  // optional counters
 };
 int fgc_launch_knn(const KnnArgs &a, hipStream_t s);

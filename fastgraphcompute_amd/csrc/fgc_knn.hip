@@ -554,15 +554,18 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                 const bool is_self = I[s] == self;
                 a.out_idx[orig_q * K + slot] = is_self ? orig_q : (long long)a.order[I[s]];
                 a.out_dist[orig_q * K + slot] = is_self ? 0.f : L[s];
+                if (a.out_sorted) a.out_sorted[(long long)self * K + slot] = I[s];
             }
             const int pslot = s * 64 + lane;      // padding slots and, if needed, the query's own slot 0
             if (pslot < K && pslot >= n_out) {
                 a.out_idx[orig_q * K + pslot] = a.tf_compat ? orig_q : -1ll;
                 a.out_dist[orig_q * K + pslot] = 0.f;
+                if (a.out_sorted) a.out_sorted[(long long)self * K + pslot] = -1;
             }
             if (!has_self && pslot == 0) {
                 a.out_idx[orig_q * K] = orig_q;
                 a.out_dist[orig_q * K] = 0.f;
+                if (a.out_sorted) a.out_sorted[(long long)self * K] = self;
             }
         }
     }

@@ -192,6 +192,174 @@ extern "C" int fgc_binned_select_knn_grad_f32(const float *d_grad_distsq, const 
 }
 
 // ---------------------------------------------------------------------------
+// the same gradient from the search's sorted-space neighbour rows
+// ---------------------------------------------------------------------------
+// The kernel above gathers x[m] from the original order, where the neighbours of a query sit in 64 different
+// cache lines: 64 M gathers pull 8 GB of lines out of L2 for 0.8 GB of payload, and that transfer is what bounds
+// it.  In the search's sorted order neighbours are memory neighbours.  This variant reads the neighbour rows the
+// search wrote in that order (int32, streaming), a padded array-of-points copy of the coordinates in the same
+// order (one 16-byte gather per neighbour and four coordinates), and only the upstream gradient row and the
+// final atomics go through the permutation.
+__global__ __launch_bounds__(256) void k_sorted_points(const float *__restrict__ x, const uint32_t *__restrict__ order,
+                                                       int64_t n, int D, int D4, float4 *__restrict__ xs)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n * D4) return;
+    const int64_t r = t / D4;
+    const int c4 = (int)(t - r * D4);
+    const int64_t o = order[r];
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] = (c4 * 4 + e < D) ? x[o * D + c4 * 4 + e] : 0.f;
+    xs[t] = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+__global__ __launch_bounds__(256) void k_knn_grad_sorted(const float *__restrict__ gd, const int *__restrict__ nbr,
+                                                         const float4 *__restrict__ xs,
+                                                         const uint32_t *__restrict__ order, float *__restrict__ gx,
+                                                         int64_t n, int K, int D, int H, int *__restrict__ status)
+{
+    extern __shared__ __align__(16) unsigned char s_raw[];
+    const int lane = fgc_lane();
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int D4 = (D + 3) >> 2;
+    const size_t wave_bytes = (size_t)H * (4 + 16 * (size_t)D4);
+    float4 *vals = (float4 *)(s_raw + wave_bytes * wv);
+    unsigned *keys = (unsigned *)(s_raw + wave_bytes * wv + (size_t)H * 16 * D4);
+    for (int t = lane; t < H; t += 64) keys[t] = GRAD_EMPTY;
+    for (int t = lane; t < H * D4; t += 64) vals[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const unsigned hmask = (unsigned)H - 1u;
+    bool bad = false;
+    auto slot_of = [&](unsigned m) -> int {
+        unsigned h = (m * 2654435761u) >> 7;
+        for (int p = 0; p < GRAD_PROBES; p++) {
+            const unsigned sl = (h + p) & hmask;
+            const unsigned old = atomicCAS(&keys[sl], GRAD_EMPTY, m);
+            if (old == GRAD_EMPTY || old == m) return (int)sl;
+        }
+        return -1;
+    };
+
+    const int64_t wave0 = ((int64_t)blockIdx.x * 4 + wv) * GW;
+    for (int q0 = 0; q0 < GW; q0 += GU) {
+        int64_t r[GU], qo[GU];
+        bool qv[GU];
+#pragma unroll
+        for (int u = 0; u < GU; u++) {
+            r[u] = wave0 + q0 + u;
+            qv[u] = r[u] < n;
+            if (!qv[u]) r[u] = 0;
+            qo[u] = order[r[u]];
+        }
+        for (int k0 = 0; k0 < K; k0 += 64) {
+            const int k = k0 + lane;
+            int m[GU], sl[GU];
+            float g[GU];
+#pragma unroll
+            for (int u = 0; u < GU; u++) {
+                m[u] = -1; g[u] = 0.f;
+                if (k < K && qv[u]) { m[u] = nbr[r[u] * K + k]; g[u] = gd[qo[u] * K + k]; }
+            }
+#pragma unroll
+            for (int u = 0; u < GU; u++) {
+                if (m[u] >= n) { bad = true; m[u] = -1; }
+                sl[u] = (m[u] >= 0) ? slot_of((unsigned)m[u]) : -1;
+            }
+            for (int c4 = 0; c4 < D4; c4++) {
+#pragma unroll
+                for (int u = 0; u < GU; u++) {
+                    const float4 xi = xs[r[u] * D4 + c4];
+                    float4 add = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (m[u] >= 0) {
+                        const float4 xm = xs[(int64_t)m[u] * D4 + c4];
+                        const float g2 = 2.f * g[u];
+                        add = make_float4(g2 * (xm.x - xi.x), g2 * (xm.y - xi.y), g2 * (xm.z - xi.z), g2 * (xm.w - xi.w));
+                    }
+                    float self[4];
+                    self[0] = fgc_wave_sum(add.x);
+                    self[1] = (c4 * 4 + 1 < D) ? fgc_wave_sum(add.y) : 0.f;
+                    self[2] = (c4 * 4 + 2 < D) ? fgc_wave_sum(add.z) : 0.f;
+                    self[3] = (c4 * 4 + 3 < D) ? fgc_wave_sum(add.w) : 0.f;
+                    if (m[u] >= 0) {
+                        if (sl[u] >= 0) {
+                            float4 v = vals[sl[u] * D4 + c4];
+                            v.x += add.x; v.y += add.y; v.z += add.z; v.w += add.w;
+                            vals[sl[u] * D4 + c4] = v;
+                        } else {
+                            const int64_t mo = order[m[u]];
+                            if (c4 * 4 + 0 < D) atomicAdd(&gx[mo * D + c4 * 4 + 0], add.x);
+                            if (c4 * 4 + 1 < D) atomicAdd(&gx[mo * D + c4 * 4 + 1], add.y);
+                            if (c4 * 4 + 2 < D) atomicAdd(&gx[mo * D + c4 * 4 + 2], add.z);
+                            if (c4 * 4 + 3 < D) atomicAdd(&gx[mo * D + c4 * 4 + 3], add.w);
+                        }
+                    }
+                    if (qv[u]) {
+                        int ss = -1;
+                        if (lane == 0) ss = slot_of((unsigned)r[u]);
+                        ss = fgc_readlane_i(ss, 0);
+                        if (lane == 0) {
+                            if (ss >= 0) {
+                                float4 v = vals[ss * D4 + c4];
+                                v.x -= self[0]; v.y -= self[1]; v.z -= self[2]; v.w -= self[3];
+                                vals[ss * D4 + c4] = v;
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 4; e++)
+                                    if (c4 * 4 + e < D) atomicAdd(&gx[qo[u] * D + c4 * 4 + e], -self[e]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+    const float *vflat = (const float *)vals;
+    for (int t = lane; t < H * D4 * 4; t += 64) {
+        const int sl = t / (D4 * 4), c = t - sl * (D4 * 4);
+        const unsigned m = keys[sl];
+        if (m == GRAD_EMPTY || c >= D) continue;
+        const float v = vflat[t];
+        if (v != 0.f) atomicAdd(&gx[(int64_t)order[m] * D + c], v);
+    }
+    if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
+}
+
+extern "C" size_t fgc_binned_select_knn_grad_sorted_workspace_bytes(int64_t n_vert, int32_t n_coords)
+{
+    if (n_vert < 0 || n_coords < 1) return 0;
+    return fgc_align((size_t)(n_vert > 0 ? n_vert : 1) * (size_t)((n_coords + 3) / 4) * 16);
+}
+
+extern "C" int fgc_binned_select_knn_grad_sorted_f32(const float *d_grad_distsq, const int32_t *d_nbr_sorted,
+                                                     const float *d_coords, const int32_t *d_order,
+                                                     float *d_grad_coords, int64_t n_vert, int32_t K,
+                                                     int32_t n_coords, int32_t *d_status, void *d_ws,
+                                                     size_t ws_bytes, void *stream)
+{
+    if (n_vert < 0 || K < 1 || n_coords < 1 || n_coords > 128) return FGC_EINVAL;
+    if (n_vert >= (1ll << 31) - 1) return FGC_EINVAL;
+    if (n_vert == 0) return FGC_OK;
+    if (!d_grad_distsq || !d_nbr_sorted || !d_coords || !d_order || !d_grad_coords) return FGC_EINVAL;
+    if (!d_ws || ws_bytes < fgc_binned_select_knn_grad_sorted_workspace_bytes(n_vert, n_coords)) return FGC_ENOSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    int rc = fgc_fill_u32(d_grad_coords, 0u, n_vert * n_coords, s);
+    if (rc) return rc;
+    const int D4 = (n_coords + 3) / 4;
+    float4 *xs = (float4 *)d_ws;
+    hipLaunchKernelGGL(k_sorted_points, dim3((unsigned)fgc_cdiv(n_vert * D4, 256)), dim3(256), 0, s, d_coords,
+                       (const uint32_t *)d_order, n_vert, (int)n_coords, D4, xs);
+    FGC_LAUNCH_CHECK();
+    const int H = grad_table_size(n_coords);
+    const size_t lds = 4 * (size_t)H * (4 + 16 * (size_t)D4);
+    const unsigned blocks = (unsigned)fgc_cdiv(n_vert, 4 * GW);
+    hipLaunchKernelGGL(k_knn_grad_sorted, dim3(blocks), dim3(256), lds, s, d_grad_distsq, d_nbr_sorted,
+                       (const float4 *)xs, (const uint32_t *)d_order, d_grad_coords, n_vert, (int)K, (int)n_coords, H,
+                       d_status);
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
+}
+
+// ---------------------------------------------------------------------------
 // select_with_default
 // ---------------------------------------------------------------------------
 // T is the element as a bit pattern (uint32_t for float / int32, uint64_t for int64 / double).

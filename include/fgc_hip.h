@@ -132,7 +132,11 @@ int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_c
  * prepare = geometry + binning + sort + bin boundaries + sorted coordinate
  * copy (binned_knn_autograd_kernel.cpp:100-139); search = the neighbour
  * search with the un-sort fused (:157-195).  Both take the same shape
- * arguments; the workspace must not be touched in between. */
+ * arguments; the workspace must not be touched in between.  d_nbr_sorted
+ * (optional, int32 [n_vert, K]) receives the neighbour rows once more in the
+ * search's own sorted order - row r belongs to the r-th point of that order and
+ * holds positions in it, -1 padding - which is the layout
+ * fgc_binned_select_knn_grad_sorted_f32 reads. */
 int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
                                const int64_t *d_row_splits, const int64_t *row_splits_host,
                                int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
@@ -141,8 +145,8 @@ int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert, int32_t n_
 int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
                               int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
                               int32_t with_direction, int32_t tf_compat, int64_t *d_idx,
-                              float *d_distsq, uint64_t *d_stats, void *d_ws, size_t ws_bytes,
-                              void *stream);
+                              float *d_distsq, int32_t *d_nbr_sorted, uint64_t *d_stats, void *d_ws,
+                              size_t ws_bytes, void *stream);
 
 /* ---------------------------------------------------------------------------
  * k nearest neighbours inside a radius.  Replaces select_knn_cuda_fn
@@ -194,6 +198,16 @@ int fgc_binned_knn_export_order_i32(int64_t n_vert, int32_t n_coords, const int6
                                     int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
                                     int32_t with_direction, const void *d_ws, size_t ws_bytes,
                                     int32_t *d_order_out, void *stream);
+
+/* The same gradient from the neighbour rows in the search's sorted order (d_nbr_sorted as written by
+ * fgc_binned_knn_search_f32, d_order as exported by fgc_binned_knn_export_order_i32): neighbours are then memory
+ * neighbours, which is what makes the coordinate gathers cheap.  d_grad_distsq, d_coords and d_grad_coords stay
+ * in the original order.  d_ws: fgc_binned_select_knn_grad_sorted_workspace_bytes(n_vert, n_coords) bytes. */
+size_t fgc_binned_select_knn_grad_sorted_workspace_bytes(int64_t n_vert, int32_t n_coords);
+int fgc_binned_select_knn_grad_sorted_f32(const float *d_grad_distsq, const int32_t *d_nbr_sorted,
+                                          const float *d_coords, const int32_t *d_order, float *d_grad_coords,
+                                          int64_t n_vert, int32_t K, int32_t n_coords, int32_t *d_status,
+                                          void *d_ws, size_t ws_bytes, void *stream);
 
 /* ---------------------------------------------------------------------------
  * Replaces select_with_default (oc_helper.py:232-271) for float32 features:
