@@ -43,7 +43,7 @@ extern "C" int fgc_index_replacer_i64(const int64_t *d_in, const int64_t *d_repl
 // adjacent lanes.  Pairs that find no table slot within a few probes go to
 // global memory directly.
 #ifndef GW
-#define GW 16          // queries per wavefront
+#define GW 24          // queries per wavefront
 #endif
 #ifndef GU
 #define GU 4           // queries a wavefront processes together (loads in flight)
