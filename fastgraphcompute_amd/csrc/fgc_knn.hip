@@ -535,15 +535,39 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             valid[0] = lane < c;                  // the c finite keys are now in lanes 0..c-1
             rank[0] = lane;
         } else {
-            // rank sort: position = number of entries that precede (by distance, then slot)
-            for (int e = 0; e < c; e++) {
-                float v = 0.f;
+            // the same network over NSEG * 64 elements, element e = s * 64 + lane: partners at least 64 apart are
+            // two registers of one lane, all others sit in the same register of another lane
 #pragma unroll
-                for (int s = 0; s < NSEG; s++)
-                    if ((e >> 6) == s) v = fgc_readlane_f(L[s], e & 63);
+            for (int k = 2; k <= NSEG * 64; k <<= 1) {
 #pragma unroll
-                for (int s = 0; s < NSEG; s++) rank[s] += ((v < L[s]) || (v == L[s] && e < s * 64 + lane)) ? 1 : 0;
+                for (int jj = k >> 1; jj > 0; jj >>= 1) {
+                    if (jj >= 64) {
+#pragma unroll
+                        for (int s = 0; s < NSEG; s++) {
+                            const int s2 = s ^ (jj >> 6);
+                            if (s2 > s) {                      // each register pair once; ascending iff (e & k) == 0
+                                const bool asc = ((s * 64) & k) == 0;
+                                const bool swap = asc ? (L[s2] < L[s]) : (L[s2] > L[s]);
+                                const float d0 = swap ? L[s2] : L[s], d1 = swap ? L[s] : L[s2];
+                                const int v0 = swap ? I[s2] : I[s], v1 = swap ? I[s] : I[s2];
+                                L[s] = d0; L[s2] = d1; I[s] = v0; I[s2] = v1;
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int s = 0; s < NSEG; s++) {
+                            const float pd = __shfl_xor(L[s], jj, 64);
+                            const int pv = __shfl_xor(I[s], jj, 64);
+                            const bool keep_min = (((lane & jj) == 0) == (((s * 64 + lane) & k) == 0));
+                            const bool take = keep_min ? (pd < L[s]) : (pd > L[s]);
+                            L[s] = take ? pd : L[s];
+                            I[s] = take ? pv : I[s];
+                        }
+                    }
+                }
             }
+#pragma unroll
+            for (int s = 0; s < NSEG; s++) { valid[s] = (s * 64 + lane) < c; rank[s] = s * 64 + lane; }
         }
         const int shift = has_self ? 0 : 1;       // without the query in the pool its slot 0 is added here
         const int n_out = min(c + shift, K);
