@@ -22,7 +22,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 # HBM bytes per k_knn launch at the default workload, from two rocprofv3 --pmc runs (FETCH_SIZE x 1.99 KiB
 # + WRITE_SIZE x 1.00 KiB, factors from a plain copy kernel in the same runs)
-KNN_TRAFFIC_CFG4_BYTES = 999.4e6
+KNN_TRAFFIC_CFG4_BYTES = 1272.6e6
 
 
 def main():
@@ -151,7 +151,9 @@ def main():
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": KNN_TRAFFIC_CFG4_BYTES if (args.workload == "cfg4" and args.scale == 1.0) else None,
                 "algorithmic_bytes": bytes_alg, "distance_evaluations": c_eval,
-                "kernel_ms": round(t_knn, 4), "io_floor_bytes": 4.0 * D * n + 12.0 * K * n}
+                "kernel_ms": round(t_knn, 4),
+                # inputs + outputs of the timed launch: queries, int64 indices, distances, int32 sorted-space rows
+                "io_floor_bytes": 4.0 * D * n + 16.0 * K * n}
 
     result = {
         "metric": "kNN queries/sec and neighbours/sec at N=1M,D=3,K=64; % of HBM roofline",
