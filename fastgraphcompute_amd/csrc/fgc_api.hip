@@ -73,15 +73,22 @@ namespace {
 struct KnnCall {
     KnnWorkspace w;
     int64_t B;
-    int sub_bits;   // Morton bits per binned dimension appended to the flat bin in the sort key
+    int sub_bits;   // sub-cell bits per binned dimension appended to the flat bin in the sort key
     int key_bits;   // total significant bits of the sort key
 };
 
-// bits per binned dimension for the in-bin Morton order: as many as fit into a 32-bit key, at most 5
+// bits per binned dimension for the order inside a bin (sub-cells along a Hilbert curve): five if they fit into
+// the 32-bit key, and beyond that as many as the radix sort takes without another 8-bit pass (dense bins, e.g. a
+// cluster of 10^5 points in one bin, need the finer cells; sparse ones lose nothing)
 int choose_sub_bits(int bin_bits, int nbd)
 {
     int sb = (32 - bin_bits) / nbd;
-    if (sb > 5) sb = 5;
+    if (sb > 5) {
+        const int passes5 = (bin_bits + 5 * nbd + 7) / 8;
+        int s = 5;
+        while (s < 8 && s < sb && (bin_bits + (s + 1) * nbd + 7) / 8 == passes5) s++;
+        sb = s;
+    }
     if (sb < 0) sb = 0;
     const char *e = getenv("FGC_SUB_BITS");   // tuning override
     if (e && *e) { int v = atoi(e); if (v >= 0 && v * nbd + bin_bits <= 32) sb = v; }

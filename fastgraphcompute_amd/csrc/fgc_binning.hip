@@ -301,10 +301,12 @@ extern "C" int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t
 }
 
 // ---------------------------------------------------------------------------
-// sort keys for the kNN pipeline: key = (flat bin << sub_bits*nbd) | Morton code
-// of the point's position inside its bin (sub_bits per binned dimension).  The
-// Morton part only orders points inside a bin so that consecutive points are
-// spatially compact; it never changes which bin a point belongs to.
+// sort keys for the kNN pipeline: key = (flat bin << sub_bits*nbd) | Hilbert index
+// of the point's sub-cell inside its bin (sub_bits per binned dimension).  The
+// low part only orders points inside a bin so that consecutive points are
+// spatially compact (consecutive sub-cells of a Hilbert curve share a face, so a
+// run of 64 points has a tight bounding box wherever it starts); it never changes
+// which bin a point belongs to.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void k_bin_keys(const float *__restrict__ coords, int n, int ld, int nbd,
                                                   int sub_bits, const float *__restrict__ geom,
@@ -333,6 +335,37 @@ __global__ __launch_bounds__(256) void k_bin_keys(const float *__restrict__ coor
     }
     f += (uint32_t)event_of(rs, n_rs, v) * stride;
     if (clamped && status) atomicOr(&status[0], FGC_ST_CLAMPED);
+#ifndef FGC_MORTON_KEYS
+    // sub-cell coordinates -> transposed Hilbert index (Skilling's in-place transform: undo the excess work of
+    // the Gray code from the most significant level down, then Gray-encode), so that interleaving the bits
+    // below yields the position along a Hilbert curve through the bin's sub-cells
+    if (sub_bits > 1) {
+        const int top = 1 << (sub_bits - 1);
+        for (int q = top; q > 1; q >>= 1) {
+            const int p = q - 1;
+#pragma unroll
+            for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
+                if (d < nbd) {
+                    if (sub[d] & q) sub[0] ^= p;
+                    else { const int t = (sub[0] ^ sub[d]) & p; sub[0] ^= t; sub[d] ^= t; }
+                }
+            }
+        }
+#pragma unroll
+        for (int d = 1; d < FGC_MAX_BIN_DIMS; d++)
+            if (d < nbd) sub[d] ^= sub[d - 1];
+        int last = sub[0];
+#pragma unroll
+        for (int d = 1; d < FGC_MAX_BIN_DIMS; d++)
+            if (d < nbd) last = sub[d];
+        int t = 0;
+        for (int q = top; q > 1; q >>= 1)
+            if (last & q) t ^= q - 1;
+#pragma unroll
+        for (int d = 0; d < FGC_MAX_BIN_DIMS; d++)
+            if (d < nbd) sub[d] ^= t;
+    }
+#endif
     uint32_t code = 0;
     for (int l = sub_bits - 1; l >= 0; l--)
 #pragma unroll

@@ -17,7 +17,7 @@ int fgc_launch_gather_sorted(const float *coords, const uint32_t *order, int n, 
 struct KnnArgs {
     const float *sc;            // sorted coordinates, structure of arrays [D][ldc]
     int ldc;
-    const uint32_t *skeys;      // sorted key per point: (flat bin << key_shift) | Morton code inside the bin
+    const uint32_t *skeys;      // sorted key per point: (flat bin << key_shift) | Hilbert index inside the bin
     int key_shift;
     const float *box_lo;        // per 64-point chunk bounding boxes [D][n_chunks]
     const float *box_hi;

@@ -1,7 +1,7 @@
 // Exact k-nearest-neighbour search over bin-sorted points (gfx950, wave64).
 //
 // Work decomposition: one wavefront owns QT consecutive points of the sorted
-// order.  The order is (flat bin, Morton code inside the bin), so the queries of
+// order.  The order is (flat bin, Hilbert index inside the bin), so the queries of
 // a wavefront are spatial neighbours and every 64 consecutive points ("chunk")
 // form a compact cluster whose bounding box is precomputed.
 //
