@@ -88,11 +88,11 @@ def test_own_search_grid_host():
     from fastgraphcompute_amd.workloads import cfg5_many_events_d8
     from fastgraphcompute_amd._ops import choose_search_grid
     t = lambda v: torch.tensor(v, dtype=torch.int64)
-    assert choose_search_grid(t([0, 1000000]), 3, 3) == (3, 26)          # ~24 chunks of 64 points per bin row
-    assert choose_search_grid(t([0, 50000, 100000, 150000, 200000]), 4, 3) == (4, 3)
-    assert choose_search_grid(t([0, 200000]), 4, 3) == (4, 5)
-    assert choose_search_grid(torch.from_numpy(cfg5_many_events_d8()["row_splits"]).long(), 8, 3) == (4, 2)
-    assert choose_search_grid(t([0, 6000, 10000]), 3, 3) == (3, 2)
+    assert choose_search_grid(t([0, 1000000]), 3, 3) == (3, 12)          # ~100 chunks of 64 points per bin row
+    assert choose_search_grid(t([0, 50000, 100000, 150000, 200000]), 4, 3) == (4, 2)
+    assert choose_search_grid(t([0, 200000]), 4, 3) == (4, 3)
+    assert choose_search_grid(torch.from_numpy(cfg5_many_events_d8()["row_splits"]).long(), 8, 3) == (4, 1)
+    assert choose_search_grid(t([0, 6000, 10000]), 3, 3) == (3, 1)
     assert choose_search_grid(t([0, 10]), 2, 3) == (2, 1)
     assert choose_search_grid(t([0, 100000000]), 2, 2) == (2, 30)       # capped
 
