@@ -27,6 +27,37 @@ extern "C" int fgc_index_replacer_i64(const int64_t *d_in, const int64_t *d_repl
     return FGC_OK;
 }
 
+// Overflow of the per-wavefront table: the lanes flagged `ovf` add their float4 `add` to the four coordinates
+// c0 .. c0 + 3 of row `target` of gx.  With more than a few such lanes the values are exchanged between the lanes
+// so that each atomic instruction carries 16 targets with their four coordinates in adjacent lanes: the memory
+// side then sees one 16-byte update per target instead of one per coordinate, and it is the number of such
+// updates that bounds the atomic rate.  Wave-uniform call (all lanes, same c0).
+__device__ __forceinline__ void grad_overflow_add(unsigned long long ovf_mask, bool ovf, int target, float4 add,
+                                                  int c0, int D, float *__restrict__ gx, int lane)
+{
+    if (__popcll(ovf_mask) <= 6) {
+        if (ovf) {
+            if (c0 + 0 < D) atomicAdd(&gx[(int64_t)target * D + c0 + 0], add.x);
+            if (c0 + 1 < D) atomicAdd(&gx[(int64_t)target * D + c0 + 1], add.y);
+            if (c0 + 2 < D) atomicAdd(&gx[(int64_t)target * D + c0 + 2], add.z);
+            if (c0 + 3 < D) atomicAdd(&gx[(int64_t)target * D + c0 + 3], add.w);
+        }
+        return;
+    }
+    const int tgt = ovf ? target : -1;
+    const int comp = lane & 3;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        if (!((ovf_mask >> (16 * r)) & 0xffffull)) continue;   // none of these 16 lanes overflowed
+        const int e = r * 16 + (lane >> 2);
+        const int te = __shfl(tgt, e, 64);
+        const float v0 = __shfl(add.x, e, 64), v1 = __shfl(add.y, e, 64);
+        const float v2 = __shfl(add.z, e, 64), v3 = __shfl(add.w, e, 64);
+        const float v = comp == 0 ? v0 : comp == 1 ? v1 : comp == 2 ? v2 : v3;
+        if (te >= 0 && c0 + comp < D) atomicAdd(&gx[(int64_t)te * D + c0 + comp], v);
+    }
+}
+
 // ---------------------------------------------------------------------------
 // gradient of distsq wrt the coordinates
 // ---------------------------------------------------------------------------
@@ -118,18 +149,17 @@ __global__ __launch_bounds__(256) void k_knn_grad(const float *__restrict__ gd, 
                         if (c < D && m[u] >= 0) add[e] = 2.f * g[u] * (x[m[u] * D + c] - x[qi[u] * D + c]);
                         self[e] = (c < D) ? fgc_wave_sum(add[e]) : 0.f;
                     }
-                    if (m[u] >= 0) {
-                        if (sl[u] >= 0) {
-                            // distinct targets within the instruction, private table: plain read-add-write
-                            float4 v = vals[sl[u] * D4 + c4];
-                            v.x += add[0]; v.y += add[1]; v.z += add[2]; v.w += add[3];
-                            vals[sl[u] * D4 + c4] = v;
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; e++)
-                                if (c4 * 4 + e < D) atomicAdd(&gx[m[u] * D + c4 * 4 + e], add[e]);
-                        }
+                    if (m[u] >= 0 && sl[u] >= 0) {
+                        // distinct targets within the instruction, private table: plain read-add-write
+                        float4 v = vals[sl[u] * D4 + c4];
+                        v.x += add[0]; v.y += add[1]; v.z += add[2]; v.w += add[3];
+                        vals[sl[u] * D4 + c4] = v;
                     }
+                    const bool ovf = m[u] >= 0 && sl[u] < 0;
+                    const unsigned long long om = fgc_ballot(ovf);
+                    if (om)
+                        grad_overflow_add(om, ovf, (int)m[u], make_float4(add[0], add[1], add[2], add[3]), c4 * 4, D,
+                                          gx, lane);
                     // the query's own share, after the neighbours' updates of this instruction
                     if (qv[u]) {
                         int ss = -1;
@@ -280,19 +310,14 @@ __global__ __launch_bounds__(256) void k_knn_grad_sorted(const float *__restrict
                     self[1] = (c4 * 4 + 1 < D) ? fgc_wave_sum(add.y) : 0.f;
                     self[2] = (c4 * 4 + 2 < D) ? fgc_wave_sum(add.z) : 0.f;
                     self[3] = (c4 * 4 + 3 < D) ? fgc_wave_sum(add.w) : 0.f;
-                    if (m[u] >= 0) {
-                        if (sl[u] >= 0) {
-                            float4 v = vals[sl[u] * D4 + c4];
-                            v.x += add.x; v.y += add.y; v.z += add.z; v.w += add.w;
-                            vals[sl[u] * D4 + c4] = v;
-                        } else {
-                            const int64_t mo = order[m[u]];
-                            if (c4 * 4 + 0 < D) atomicAdd(&gx[mo * D + c4 * 4 + 0], add.x);
-                            if (c4 * 4 + 1 < D) atomicAdd(&gx[mo * D + c4 * 4 + 1], add.y);
-                            if (c4 * 4 + 2 < D) atomicAdd(&gx[mo * D + c4 * 4 + 2], add.z);
-                            if (c4 * 4 + 3 < D) atomicAdd(&gx[mo * D + c4 * 4 + 3], add.w);
-                        }
+                    if (m[u] >= 0 && sl[u] >= 0) {
+                        float4 v = vals[sl[u] * D4 + c4];
+                        v.x += add.x; v.y += add.y; v.z += add.z; v.w += add.w;
+                        vals[sl[u] * D4 + c4] = v;
                     }
+                    const bool ovf = m[u] >= 0 && sl[u] < 0;
+                    const unsigned long long om = fgc_ballot(ovf);
+                    if (om) grad_overflow_add(om, ovf, ovf ? (int)order[m[u]] : -1, add, c4 * 4, D, gx, lane);
                     if (qv[u]) {
                         int ss = -1;
                         if (lane == 0) ss = slot_of((unsigned)r[u]);
