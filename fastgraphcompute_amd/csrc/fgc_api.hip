@@ -90,8 +90,6 @@ int choose_sub_bits(int bin_bits, int nbd)
         sb = s;
     }
     if (sb < 0) sb = 0;
-    const char *e = getenv("FGC_SUB_BITS");   // tuning override
-    if (e && *e) { int v = atoi(e); if (v >= 0 && v * nbd + bin_bits <= 32) sb = v; }
     return sb;
 }
 
