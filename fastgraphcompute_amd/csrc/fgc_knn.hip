@@ -52,8 +52,8 @@
 #ifndef PRUNE_MARGIN
 #define PRUNE_MARGIN 24 // a pool is pruned when fewer than this many slots are free
 #endif
-#ifndef SEED_W
-#define SEED_W 1     // seed chunks on either side of the wavefront's own chunk, per 64 neighbours asked for
+#ifndef SEED_K
+#define SEED_K 40    // one seed chunk on either side of the wavefront's own chunk per this many neighbours asked for
 #endif
 #ifndef CULL_MIN
 #define CULL_MIN 5     // spans of at least this many chunks get the per-chunk box test
@@ -247,8 +247,9 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
         const int evrow0 = ev * rows_per_event;
         const int ev_j0 = bb[evrow0 * nz], ev_j1 = bb[(evrow0 + rows_per_event) * nz];
         const int own = qbeg >> 6;
-        const int seed_c0 = max(own - SEED_W * NSEG, ev_j0 >> 6);
-        const int seed_c1 = min(own + SEED_W * NSEG, (ev_j1 - 1) >> 6);
+        const int seed_w = (K + SEED_K - 1) / SEED_K;
+        const int seed_c0 = max(own - seed_w, ev_j0 >> 6);
+        const int seed_c1 = min(own + seed_w, (ev_j1 - 1) >> 6);
 
         // span iteration state: phase 0 = own chunk, 1 = the other seed chunks, 2 = bin rows ring by ring
         int phase = 0, d = 0;
