@@ -59,6 +59,80 @@
 #define CULL_MIN 5     // spans of at least this many chunks get the per-chunk box test
 #endif
 
+// ---- bitonic network across the lanes without LDS traffic ----
+// partner value for lane ^ JJ: DPP moves inside a row of 16 lanes, the lane-swap instructions of gfx950 across rows
+__device__ __forceinline__ int fgc_sel_i(unsigned long long mask, int if_set, int if_clear)
+{
+    int r;
+    asm volatile("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(if_clear), "v"(if_set), "s"(mask));
+    return r;
+}
+template <int JJ> __device__ __forceinline__ int fgc_xor_lane(int v)
+{
+    if constexpr (JJ == 1) return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, true);        // quad_perm [1,0,3,2]
+    else if constexpr (JJ == 2) return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
+    else if constexpr (JJ == 4) {
+        const int t = __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, true);                   // row_half_mirror: ^7
+        return __builtin_amdgcn_update_dpp(0, t, 0x1B, 0xf, 0xf, true);                           // quad_perm [3,2,1,0]: ^3
+    } else if constexpr (JJ == 8) return __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, true);  // row_ror:8
+    else if constexpr (JJ == 16) {
+        // odd rows of the first operand are swapped with the even rows of the second
+        const auto r = __builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false);
+        return fgc_sel_i(0xffff0000ffff0000ull, (int)r[0], (int)r[1]);
+    } else {
+        // upper half of the first operand is swapped with the lower half of the second
+        const auto r = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);
+        return fgc_sel_i(0xffffffff00000000ull, (int)r[0], (int)r[1]);
+    }
+}
+// lanes that keep the smaller key in the step (k, jj) of the network over elements e = s * 64 + lane
+constexpr unsigned long long fgc_keep_min_mask(int k, int jj, int s)
+{
+    unsigned long long m = 0;
+    for (int l = 0; l < 64; l++) {
+        const int e = s * 64 + l;
+        if (((e & jj) == 0) == ((e & k) == 0)) m |= 1ull << l;
+    }
+    return m;
+}
+// one compare-exchange step with partners jj < 64 lanes apart; equal keys never move
+template <int KK, int JJ, int NSEG> __device__ __forceinline__ void fgc_bitonic_step(float (&L)[NSEG], int (&I)[NSEG])
+{
+#pragma unroll
+    for (int s = 0; s < NSEG; s++) {
+        const unsigned long long km = fgc_keep_min_mask(KK, JJ, s);
+        const float pd = __int_as_float(fgc_xor_lane<JJ>(__float_as_int(L[s])));
+        const int pv = fgc_xor_lane<JJ>(I[s]);
+        const unsigned long long lt = fgc_ballot(pd < L[s]), gt = fgc_ballot(pd > L[s]);
+        const unsigned long long take = (lt & km) | (gt & ~km);
+        L[s] = __int_as_float(fgc_sel_i(take, __float_as_int(pd), __float_as_int(L[s])));
+        I[s] = fgc_sel_i(take, pv, I[s]);
+    }
+}
+template <int KK, int JJ, int NSEG> struct FgcBitonic {
+    static __device__ __forceinline__ void run(float (&L)[NSEG], int (&I)[NSEG])
+    {
+        if constexpr (JJ >= 64) {
+            // partners are two registers of one lane; each pair once, ascending iff (e & k) == 0
+#pragma unroll
+            for (int s = 0; s < NSEG; s++) {
+                const int s2 = s ^ (JJ >> 6);
+                if (s2 > s) {
+                    const bool asc = ((s * 64) & KK) == 0;
+                    const bool swap = asc ? (L[s2] < L[s]) : (L[s2] > L[s]);
+                    const float d0 = swap ? L[s2] : L[s], d1 = swap ? L[s] : L[s2];
+                    const int v0 = swap ? I[s2] : I[s], v1 = swap ? I[s] : I[s2];
+                    L[s] = d0; L[s2] = d1; I[s] = v0; I[s2] = v1;
+                }
+            }
+        } else {
+            fgc_bitonic_step<KK, JJ, NSEG>(L, I);
+        }
+        if constexpr (JJ > 1) FgcBitonic<KK, JJ / 2, NSEG>::run(L, I);
+        else if constexpr (KK < NSEG * 64) FgcBitonic<KK * 2, KK, NSEG>::run(L, I);
+    }
+};
+
 // wavefronts per block, chosen so that a block's pools fit the 64 KB static LDS limit
 // one wavefront per block: no block-level cooperation is used, and small blocks pack the LDS of a CU best
 template <int NSEG> struct KnnCfg { static constexpr int WPB = 1; };
@@ -495,13 +569,15 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
         }
     }
 
-    // ---- per query: cut the pool to exactly K, sort by distance, write the row at the query's
+    // ---- per query: sort the pool by distance, write its first K entries as the row at the query's
     //      original position (slot 0 = the query itself) ----
     for (int q = 0; q < nq; q++) {
         const int self = qbeg + q;
         const long long orig_q = (long long)a.order[self];
-        prune(q, true);
-        const int c = fgc_readlane_i(cnt, q);     // <= K entries now, compacted in slots 0..c-1
+        // the sort below takes NSEG * 64 entries: a pool that fits is sorted as it is and its first K entries are
+        // written, a larger one is first cut to exactly K
+        if (fgc_readlane_i(cnt, q) > NSEG * 64) prune(q, true);
+        const int c = fgc_readlane_i(cnt, q);     // entries in slots 0..c-1, c <= NSEG * 64
         float L[NSEG];
         int I[NSEG], rank[NSEG];
         bool valid[NSEG];
@@ -516,60 +592,12 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             has_self = has_self || (fgc_ballot(is_self) != 0ull);
             rank[s] = 0;
         }
-        if (NSEG == 1) {
-            // bitonic sort of the 64 (distance, index) pairs across the lanes; equal keys never swap
-            float kd = L[0];
-            int kv = I[0];
+        // bitonic sort of the NSEG * 64 (distance, index) pairs, element e = s * 64 + lane; equal keys never swap.
+        // Partners less than 64 apart sit in the same register of another lane, the others are two registers of
+        // one lane.  The c finite keys end up in elements 0 .. c-1.
+        FgcBitonic<2, 1, NSEG>::run(L, I);
 #pragma unroll
-            for (int k = 2; k <= 64; k <<= 1) {
-#pragma unroll
-                for (int jj = k >> 1; jj > 0; jj >>= 1) {
-                    const float pd = __shfl_xor(kd, jj, 64);
-                    const int pv = __shfl_xor(kv, jj, 64);
-                    const bool keep_min = (((lane & jj) == 0) == ((lane & k) == 0));
-                    const bool take = keep_min ? (pd < kd) : (pd > kd);
-                    kd = take ? pd : kd;
-                    kv = take ? pv : kv;
-                }
-            }
-            L[0] = kd; I[0] = kv;
-            valid[0] = lane < c;                  // the c finite keys are now in lanes 0..c-1
-            rank[0] = lane;
-        } else {
-            // the same network over NSEG * 64 elements, element e = s * 64 + lane: partners at least 64 apart are
-            // two registers of one lane, all others sit in the same register of another lane
-#pragma unroll
-            for (int k = 2; k <= NSEG * 64; k <<= 1) {
-#pragma unroll
-                for (int jj = k >> 1; jj > 0; jj >>= 1) {
-                    if (jj >= 64) {
-#pragma unroll
-                        for (int s = 0; s < NSEG; s++) {
-                            const int s2 = s ^ (jj >> 6);
-                            if (s2 > s) {                      // each register pair once; ascending iff (e & k) == 0
-                                const bool asc = ((s * 64) & k) == 0;
-                                const bool swap = asc ? (L[s2] < L[s]) : (L[s2] > L[s]);
-                                const float d0 = swap ? L[s2] : L[s], d1 = swap ? L[s] : L[s2];
-                                const int v0 = swap ? I[s2] : I[s], v1 = swap ? I[s] : I[s2];
-                                L[s] = d0; L[s2] = d1; I[s] = v0; I[s2] = v1;
-                            }
-                        }
-                    } else {
-#pragma unroll
-                        for (int s = 0; s < NSEG; s++) {
-                            const float pd = __shfl_xor(L[s], jj, 64);
-                            const int pv = __shfl_xor(I[s], jj, 64);
-                            const bool keep_min = (((lane & jj) == 0) == (((s * 64 + lane) & k) == 0));
-                            const bool take = keep_min ? (pd < L[s]) : (pd > L[s]);
-                            L[s] = take ? pd : L[s];
-                            I[s] = take ? pv : I[s];
-                        }
-                    }
-                }
-            }
-#pragma unroll
-            for (int s = 0; s < NSEG; s++) { valid[s] = (s * 64 + lane) < c; rank[s] = s * 64 + lane; }
-        }
+        for (int s = 0; s < NSEG; s++) { valid[s] = (s * 64 + lane) < c; rank[s] = s * 64 + lane; }
         const int shift = has_self ? 0 : 1;       // without the query in the pool its slot 0 is added here
         const int n_out = min(c + shift, K);
 #pragma unroll
