@@ -145,7 +145,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     constexpr int PS = NSEG + 1;          // pool segments (lanes x PS cover the pool)
     constexpr int WPB = KnnCfg<NSEG>::WPB;
     constexpr int DR = DT > 0 ? DT : 1;
-    extern __shared__ float s_pool[];     // [WPB][2][QT * CAP]: distances, then sorted positions (as int)
+    extern __shared__ uint2 s_pool[];     // [WPB][QT * CAP] (distance bits, sorted position): one 8-byte LDS access per entry
     const int CAP = a.pool_cap;           // pool capacity per query: K kept + room for new candidates
 
     const int lane = fgc_lane();
@@ -155,8 +155,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     const int qbeg = (blockIdx.x * WPB + wv) * QT;
     if (qbeg >= a.n) return;  // no block-wide barrier is used below
     const int nq = min(QT, a.n - qbeg);
-    float *ld = s_pool + (size_t)wv * 2 * QT * CAP;
-    int *li = (int *)(ld + QT * CAP);
+    uint2 *pool = s_pool + (size_t)wv * QT * CAP;
 
     const int K = a.K, nbd = a.nbd, ldc = a.ldc, nch = a.n_chunks;
     const float *__restrict__ sc = a.sc;
@@ -218,8 +217,9 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 #pragma unroll
         for (int s = 0; s < PS; s++) {
             const bool valid = (s * 64 + lane) < c;
-            P[s] = valid ? __float_as_uint(ld[q * CAP + s * 64 + lane]) : 0xffffffffu;
-            PI[s] = valid ? li[q * CAP + s * 64 + lane] : -1;
+            const uint2 e = valid ? pool[q * CAP + s * 64 + lane] : make_uint2(0xffffffffu, 0xffffffffu);
+            P[s] = e.x;
+            PI[s] = (int)e.y;
         }
         auto count_le = [&](unsigned t) -> int {
             int n = 0;
@@ -285,8 +285,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             const unsigned long long km = fgc_ballot(keep[s]);
             if (keep[s]) {
                 const int pos = base + fgc_mbcnt(km);
-                ld[q * CAP + pos] = __uint_as_float(P[s]);
-                li[q * CAP + pos] = PI[s];
+                pool[q * CAP + pos] = make_uint2(P[s], (unsigned)PI[s]);
             }
             base += __popcll(km);
         }
@@ -536,7 +535,8 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                                 }
                             }
                         }
-                        unsigned long long pm = fgc_ballot(dsq < t);
+                        bool want = dsq < t;               // lanes whose candidate still has to go into the pool
+                        unsigned long long pm = fgc_ballot(want);
                         if (!pm) continue;
                         CNT(n_app++);
                         // ---- append the passing lanes to query q's pool; when it overflows or runs nearly
@@ -546,10 +546,9 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                         for (int attempt = 0;; attempt++) {
                             const int room = CAP - pc;
                             const int rnk = fgc_mbcnt(pm);
-                            const bool put = ((pm >> lane) & 1ull) && rnk < room;
+                            const bool put = want && rnk < room;
                             if (put) {
-                                ld[q * CAP + pc + rnk] = dsq;
-                                li[q * CAP + pc + rnk] = j;
+                                pool[q * CAP + pc + rnk] = make_uint2(__float_as_uint(dsq), (unsigned)j);
                             }
                             const int npm = __popcll(pm);
                             pc += min(npm, room);
@@ -560,7 +559,8 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                             prune(q, attempt > 0);
                             if (!left) break;
                             pc = fgc_readlane_i(cnt, q);
-                            pm = fgc_ballot(((pm >> lane) & 1ull) && rnk >= room && dsq < fgc_readlane_f(tau, q));
+                            want = want && rnk >= room && dsq < fgc_readlane_f(tau, q);
+                            pm = fgc_ballot(want);
                             if (!pm) break;
                         }
                     }
@@ -585,8 +585,9 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 #pragma unroll
         for (int s = 0; s < NSEG; s++) {
             valid[s] = (s * 64 + lane) < c;
-            L[s] = valid[s] ? ld[q * CAP + s * 64 + lane] : INFINITY;
-            I[s] = valid[s] ? li[q * CAP + s * 64 + lane] : -1;
+            const uint2 e = valid[s] ? pool[q * CAP + s * 64 + lane] : make_uint2(0x7f800000u, 0xffffffffu);
+            L[s] = __uint_as_float(e.x);
+            I[s] = (int)e.y;
             const bool is_self = valid[s] && I[s] == self;
             if (is_self) L[s] = -1.f;             // the query itself sorts first
             has_self = has_self || (fgc_ballot(is_self) != 0ull);
