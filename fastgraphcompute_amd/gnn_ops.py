@@ -26,6 +26,31 @@ def dense(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -
     return torch.ops.fastgraphcompute_custom_ops.dense(x, weight, bias)
 
 
+class Dense(torch.nn.Linear):
+    """torch.nn.Linear (same parameters, state_dict and results) whose weight gradient is the library's split
+    reduction over the points.  For the layers around GravNetOp in a point-cloud model: their weight-gradient
+    products have 10^5..10^6 rows and an output of at most a few hundred squared, the shape on which a tiled
+    library GEMM leaves most of the chip idle."""
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        return dense(input, self.weight, self.bias)
+
+
+def use_dense_layers(module: torch.nn.Module) -> torch.nn.Module:
+    """Replaces every plain torch.nn.Linear inside `module` by a Dense layer sharing its parameters (in place;
+    optimizers and state_dicts built on the parameters stay valid).  Returns `module`."""
+    for name, child in module.named_children():
+        if type(child) is torch.nn.Linear:
+            layer = Dense(child.in_features, child.out_features, bias=child.bias is not None,
+                          device=child.weight.device, dtype=child.weight.dtype)
+            layer.weight = child.weight
+            layer.bias = child.bias
+            setattr(module, name, layer)
+        else:
+            use_dense_layers(child)
+    return module
+
+
 class GravNetOp(torch.nn.Module):
     """One GravNet layer [arxiv:1902.07987]: learned coordinates -> kNN graph ->
     exp(-10 d^2)-weighted mean/max aggregation of learned features -> dense output."""

@@ -88,3 +88,30 @@ def test_gravnet_weight_gradients_against_float64():
             else float(ref.abs().max())
         assert float((got[k] - ref).abs().max()) < 2e-4 * scale, k
     assert float((gx - xd.grad).abs().max()) < 2e-4 * float(xd.grad.abs().max())
+
+
+def test_use_dense_layers_keeps_results_and_parameters():
+    """A model with its nn.Linear layers swapped for Dense ones: same parameters (shared), outputs and gradients."""
+    from fastgraphcompute_amd.gnn_ops import Dense, use_dense_layers
+    torch.manual_seed(3)
+    model = torch.nn.Sequential(torch.nn.Linear(16, 40), torch.nn.ReLU(),
+                                torch.nn.Sequential(torch.nn.Linear(40, 40, bias=False), torch.nn.Tanh()),
+                                torch.nn.Linear(40, 3)).cuda()
+    x = torch.randn(5000, 16, device="cuda")
+    params = list(model.parameters())
+    out = model(x)
+    out.square().sum().backward()
+    ref = [p.grad.clone() for p in params]
+    model.zero_grad()
+    state = {k: v.clone() for k, v in model.state_dict().items()}
+    assert use_dense_layers(model) is model
+    assert isinstance(model[0], Dense) and isinstance(model[2][0], Dense) and isinstance(model[3], Dense)
+    assert all(a is b for a, b in zip(params, model.parameters()))          # the very same parameter tensors
+    assert list(model.state_dict().keys()) == list(state.keys())
+    out2 = model(x)
+    assert float((out2 - out).abs().max()) <= 1e-5 * float(out.abs().max())
+    out2.square().sum().backward()
+    for p, r in zip(params, ref):
+        assert float((p.grad - r).abs().max()) <= 2e-4 * float(r.abs().max())
+    scripted = torch.jit.script(model)
+    assert float((scripted(x) - out).abs().max()) <= 1e-5 * float(out.abs().max())
