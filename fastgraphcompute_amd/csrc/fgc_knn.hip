@@ -303,6 +303,33 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
         return g * g;
     };
 
+    // ---- append the lanes in `want` (candidate j at squared distance dsq, one per lane) to query q's pool; when
+    //      it overflows or runs nearly full (tau should stay tight) prune it: first to a tighter threshold, then,
+    //      if lanes are still waiting, down to exactly K ----
+    auto push = [&](int q, float dsq, int j, bool want) {
+        unsigned long long pm = fgc_ballot(want);
+        if (!pm) return;
+        CNT(n_app++);
+        int pc = fgc_readlane_i(cnt, q);
+        for (int attempt = 0;; attempt++) {
+            const int room = CAP - pc;
+            const int rnk = fgc_mbcnt(pm);
+            const bool put = want && rnk < room;
+            if (put) pool[q * CAP + pc + rnk] = make_uint2(__float_as_uint(dsq), (unsigned)j);
+            const int npm = __popcll(pm);
+            pc += min(npm, room);
+            cnt = (lane == q) ? pc : cnt;
+            const bool left = npm > room;          // lanes of rank >= room are still waiting
+            if (!left && pc <= CAP - PRUNE_MARGIN && (pc <= K || fgc_readlane_f(tau, q) < INFINITY)) break;
+            prune(q, attempt > 0);
+            if (!left) break;
+            pc = fgc_readlane_i(cnt, q);
+            want = want && rnk >= room && dsq < fgc_readlane_f(tau, q);
+            pm = fgc_ballot(want);
+            if (!pm) break;
+        }
+    };
+
     // ---- groups of queries sharing a bin row ----
     unsigned long long todo = fgc_ballot(qactive);
     while (todo) {
@@ -324,8 +351,75 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
         const int seed_c0 = max(own - seed_w, ev_j0 >> 6);
         const int seed_c1 = min(own + seed_w, (ev_j1 - 1) >> 6);
 
+        // ---- seeds in registers.  Up to SMAX chunks around the own one are held one candidate per lane; per query
+        //      their distances stay in registers, a bisection on ballot counts finds a bound with K .. K + slack of
+        //      them below it, and only those go into the pool - the query starts with a finite tau and a pool that
+        //      needs no pruning, instead of pushing every seed candidate through the pool and cutting it down two
+        //      or three times. ----
+        constexpr int SMAX = DT == 0 ? 0 : (16 / DR >= 5 ? 5 : (16 / DR >= 1 ? 16 / DR : 1));
+        int ra = own, rb = own - 1;             // register seeds: chunks ra..rb (none for DT == 0)
+        if (SMAX > 0) {
+            ra = max(seed_c0, own - (SMAX - 1) / 2);
+            rb = min(seed_c1, ra + SMAX - 1);
+            ra = max(seed_c0, rb - SMAX + 1);
+            float sx[SMAX > 0 ? SMAX : 1][DR];
+            bool sv[SMAX > 0 ? SMAX : 1];
+#pragma unroll
+            for (int s = 0; s < SMAX; s++) {
+                const int j = ((ra + s) << 6) + lane;
+                sv[s] = (ra + s <= rb) && j >= ev_j0 && j < ev_j1;
+                if (a.sdir && sv[s]) { unsigned char dd = a.sdir[j]; if (dd == 1 || dd == 2) sv[s] = false; }
+#pragma unroll
+                for (int dd = 0; dd < DR; dd++) sx[s][dd] = (ra + s <= rb && dd < a.D) ? sc[(size_t)dd * ldc + j] : 0.f;
+            }
+            nchunks += (unsigned)(rb - ra + 1);
+            for (unsigned long long m = gm; m;) {
+                const int q = __ffsll((long long)m) - 1;
+                m &= m - 1;
+                const float t0 = fgc_readlane_f(tau, q);
+                unsigned ds[SMAX > 0 ? SMAX : 1];      // distance bit patterns, 0xffffffff = no candidate
+                int total = 0;
+                unsigned mx = 0u;
+#pragma unroll
+                for (int s = 0; s < SMAX; s++) {
+                    float df = fgc_readlane_f(qx[0], q) - sx[s][0];
+                    float dsq = df * df;
+#pragma unroll
+                    for (int dd = 1; dd < DR; dd++) { df = fgc_readlane_f(qx[dd], q) - sx[s][dd]; dsq += df * df; }
+                    const bool ok = sv[s] && dsq < t0;
+                    ds[s] = ok ? __float_as_uint(dsq) : 0xffffffffu;
+                    const unsigned long long okm = fgc_ballot(ok);
+                    total += __popcll(okm);
+                    nev += (unsigned long long)__popcll(fgc_ballot(sv[s]));
+                    mx = max(mx, ok ? ds[s] : 0u);
+                }
+                unsigned sel = 0xfffffffeu;             // candidates <= sel are pushed: everything by default
+                if (total > K + slack) {
+                    float flo = 0.f, fhi = __int_as_float(fgc_wave_max_i((int)mx));
+                    for (int it = 0; it < 12; it++) {
+                        const float mid = 0.5f * (flo + fhi);
+                        int cm = 0;
+#pragma unroll
+                        for (int s = 0; s < SMAX; s++) cm += __popcll(fgc_ballot(ds[s] <= __float_as_uint(mid)));
+                        CNT(n_bis++);
+                        if (cm >= K) {
+                            fhi = mid;
+                            if (cm <= K + slack) {      // K .. K + slack seeds lie within mid: the first bound
+                                sel = __float_as_uint(mid);
+                                tau = (lane == q) ? mid : tau;
+                                break;
+                            }
+                        } else flo = mid;
+                    }
+                }
+#pragma unroll
+                for (int s = 0; s < SMAX; s++)
+                    push(q, __uint_as_float(ds[s]), ((ra + s) << 6) + lane, ds[s] <= sel);
+            }
+        }
+
         // span iteration state: phase 0 = own chunk, 1 = the other seed chunks, 2 = bin rows ring by ring
-        int phase = 0, d = 0;
+        int phase = (SMAX > 0) ? ((ra == seed_c0 && rb == seed_c1) ? 2 : 1) : 0, d = 0;
         int ai[RD], lo[RD], hi[RD];
         int zlo = 0, zhi = nz - 1;
         bool ring_open = false, ring_fresh = false, ring_any = false;
@@ -340,7 +434,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                 sk0 = 1; sk1 = 0; act = gm; phase = 1;
             } else if (phase == 1) {
                 j0 = max(ev_j0, seed_c0 << 6); j1 = min(ev_j1, (seed_c1 + 1) << 6);
-                sk0 = own; sk1 = own; act = gm; phase = 2;
+                sk0 = (SMAX > 0) ? ra : own; sk1 = (SMAX > 0) ? rb : own; act = gm; phase = 2;
             } else {
                 if (!ring_open) {
                     // start ring d: the bins the balls of radius sqrt(tau) reach (whole grid while a
@@ -535,34 +629,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                                 }
                             }
                         }
-                        bool want = dsq < t;               // lanes whose candidate still has to go into the pool
-                        unsigned long long pm = fgc_ballot(want);
-                        if (!pm) continue;
-                        CNT(n_app++);
-                        // ---- append the passing lanes to query q's pool; when it overflows or runs nearly
-                        //      full (tau should stay tight) prune it: first to a tighter threshold, then, if
-                        //      lanes are still waiting, down to exactly K ----
-                        int pc = fgc_readlane_i(cnt, q);
-                        for (int attempt = 0;; attempt++) {
-                            const int room = CAP - pc;
-                            const int rnk = fgc_mbcnt(pm);
-                            const bool put = want && rnk < room;
-                            if (put) {
-                                pool[q * CAP + pc + rnk] = make_uint2(__float_as_uint(dsq), (unsigned)j);
-                            }
-                            const int npm = __popcll(pm);
-                            pc += min(npm, room);
-                            cnt = (lane == q) ? pc : cnt;
-                            const bool left = npm > room;          // lanes of rank >= room are still waiting
-                            if (!left && pc <= CAP - PRUNE_MARGIN && (pc <= K || fgc_readlane_f(tau, q) < INFINITY))
-                                break;
-                            prune(q, attempt > 0);
-                            if (!left) break;
-                            pc = fgc_readlane_i(cnt, q);
-                            want = want && rnk >= room && dsq < fgc_readlane_f(tau, q);
-                            pm = fgc_ballot(want);
-                            if (!pm) break;
-                        }
+                        push(q, dsq, j, dsq < t);
                     }
                 }
             }
