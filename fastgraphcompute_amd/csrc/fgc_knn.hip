@@ -41,7 +41,7 @@
 #include "fgc_internal.h"
 
 #ifndef QT
-#define QT 6           // queries per wavefront (6 x 112 pool slots x 8 B = 5.4 KB of LDS: ~29 wavefronts per CU)
+#define QT 6           // queries per wavefront (6 x 128 pool slots x 8 B = 6 KB of LDS at K = 64: 26 wavefronts per CU)
 #endif
 #ifndef POOL_EXTRA
 #define POOL_EXTRA 48  // pool slots beyond K (rounded up to 16); LDS per wavefront = QT * pool slots * 8 B
@@ -64,7 +64,7 @@
 __device__ __forceinline__ int fgc_sel_i(unsigned long long mask, int if_set, int if_clear)
 {
     int r;
-    asm volatile("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(if_clear), "v"(if_set), "s"(mask));
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(if_clear), "v"(if_set), "s"(mask));
     return r;
 }
 template <int JJ> __device__ __forceinline__ int fgc_xor_lane(int v)
