@@ -10,6 +10,7 @@ Two ops have no counterpart in the reference: the fused GravNet aggregation and
 the float32 select_with_default kernel.
 """
 import struct
+import weakref
 from typing import List, Optional, Tuple
 
 import torch
@@ -196,6 +197,31 @@ def knn_grad_sorted(grad_distsq: torch.Tensor, nbr_sorted: torch.Tensor, coords:
     return out
 
 
+_RS_HOST = {}       # id(tensor) -> (weak reference, version, data pointer, host copy)
+
+
+def host_row_splits(row_splits: torch.Tensor) -> torch.Tensor:
+    """row_splits as an int64 host tensor.  The search is planned on the host, so a device tensor has to be copied
+    back, which makes the host wait for everything queued before it.  A model calls the kNN of every layer with the
+    same row_splits tensor: the copy is kept for as long as that very tensor object is alive and unmodified
+    (object identity, version counter and data pointer are all checked), so only the first call waits."""
+    if not row_splits.is_cuda:
+        return row_splits.detach().to(torch.int64).contiguous()
+    try:
+        version = row_splits._version
+    except RuntimeError:          # inference tensors have no version counter: no caching
+        return row_splits.detach().to("cpu", torch.int64).contiguous()
+    key = id(row_splits)
+    ent = _RS_HOST.get(key)
+    if ent is not None and ent[0]() is row_splits and ent[1] == version and ent[2] == row_splits.data_ptr():
+        return ent[3]
+    host = row_splits.detach().to("cpu", torch.int64).contiguous()
+    if len(_RS_HOST) >= 64:
+        _RS_HOST.clear()
+    _RS_HOST[key] = (weakref.ref(row_splits), version, row_splits.data_ptr(), host)
+    return host
+
+
 class _BinnedKNN(torch.autograd.Function):
     @staticmethod
     def forward(ctx, coords, row_splits, K, direction, n_bins, max_bin_dims, tf_compat):
@@ -213,7 +239,7 @@ class _BinnedKNN(torch.autograd.Function):
             raise ValueError("Unsupported number of binning dimensions.")
         if K < 1 or K > 256:
             raise ValueError("binned_select_knn on MI355X supports 1 <= K <= 256, got %d" % K)
-        rs_host = row_splits.detach().to("cpu", torch.int64).contiguous()
+        rs_host = host_row_splits(row_splits)
         n_rs = rs_host.numel()
         if n_rs < 2:
             raise ValueError("row_splits needs at least two entries")

@@ -267,3 +267,28 @@ def test_adversarial_distributions(oracle, name):
         for n_bins in (None, 11, 29):        # the library's own coarse grid, and fine grids with many rings
             gi, gd = _gpu_knn(K, coords, rs, n_bins=None if n_bins is None else torch.tensor(n_bins))
             assert_knn_equal(gi, gd, bi, bd, what="%s K=%d n_bins=%s" % (name, K, n_bins))
+
+
+def test_row_splits_host_copy_follows_the_tensor(oracle):
+    """The host copy of a device row_splits tensor is reused only while that very tensor is unchanged."""
+    from fastgraphcompute_amd import binned_select_knn
+    from fastgraphcompute_amd import _ops
+    rng = np.random.default_rng(77)
+    coords = rng.random((3000, 3)).astype(np.float32)
+    c = torch.from_numpy(coords).cuda()
+    rs = torch.tensor([0, 1000, 3000], dtype=torch.int64, device="cuda")
+    i1, d1 = binned_select_knn(8, c, rs)
+    n_cached = len(_ops._RS_HOST)
+    i2, d2 = binned_select_knn(8, c, rs)                  # same object: the cached copy
+    assert len(_ops._RS_HOST) == n_cached and torch.equal(i1, i2) and torch.equal(d1, d2)
+    oi, od = oracle.binned_select_knn(8, coords, np.array([0, 1000, 3000]))
+    assert_knn_equal(i1.cpu().numpy(), d1.cpu().numpy(), oi, od, what="first")
+    rs[1] = 2000                                           # in place: the version counter moves
+    i3, d3 = binned_select_knn(8, c, rs)
+    oi, od = oracle.binned_select_knn(8, coords, np.array([0, 2000, 3000]))
+    assert_knn_equal(i3.cpu().numpy(), d3.cpu().numpy(), oi, od, what="after in-place change")
+    del rs                                                 # a new tensor, whatever its address
+    rs = torch.tensor([0, 500, 3000], dtype=torch.int64, device="cuda")
+    i4, d4 = binned_select_knn(8, c, rs)
+    oi, od = oracle.binned_select_knn(8, coords, np.array([0, 500, 3000]))
+    assert_knn_equal(i4.cpu().numpy(), d4.cpu().numpy(), oi, od, what="new tensor")
