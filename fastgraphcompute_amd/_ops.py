@@ -129,14 +129,14 @@ def choose_search_grid(row_splits_host: torch.Tensor, n_coords: int, max_bin_dim
     The grid never changes the result (the search is exact), only the time.  This search prunes with the
     bounding boxes of 64-point chunks of a sort along a Hilbert curve inside each bin, so it wants far coarser bins
     than the reference's thread-per-query shell walk: up to five binned dimensions (the curve then runs through
-    all of them) and about 100 chunks per bin row, 1000 with five binned dimensions (measured optima on 2- to
+    all of them) and about 150 chunks per bin row, 300 with four and 1000 with five binned dimensions (optima on 2- to
     10-dimensional point clouds from 5 000 to 1 000 000 points per event).  With config.auto_grid = False the
     reference's heuristic (calculate_optimal_bins) and max_bin_dims are used."""
     rs = row_splits_host
     n_events = max(1, int(rs.numel()) - 1)
     n = int(torch.max(rs)) if rs.numel() > 0 else 0
     nbd = max(2, min(int(n_coords), 5))
-    rows = (n / n_events) / 64.0 / (100.0 if nbd <= 4 else 1000.0)
+    rows = (n / n_events) / 64.0 / (150.0 if nbd <= 3 else (300.0 if nbd == 4 else 1000.0))
     nb = int(round(max(rows, 1.0) ** (1.0 / (nbd - 1))))
     return nbd, max(1, min(nb, 30))
 

@@ -88,9 +88,9 @@ def test_own_search_grid_host():
     from fastgraphcompute_amd.workloads import cfg5_many_events_d8
     from fastgraphcompute_amd._ops import choose_search_grid
     t = lambda v: torch.tensor(v, dtype=torch.int64)
-    assert choose_search_grid(t([0, 1000000]), 3, 3) == (3, 12)          # ~100 chunks of 64 points per bin row
-    assert choose_search_grid(t([0, 50000, 100000, 150000, 200000]), 4, 3) == (4, 2)
-    assert choose_search_grid(t([0, 200000]), 4, 3) == (4, 3)
+    assert choose_search_grid(t([0, 1000000]), 3, 3) == (3, 10)          # ~150 chunks of 64 points per bin row
+    assert choose_search_grid(t([0, 50000, 100000, 150000, 200000]), 4, 3) == (4, 1)
+    assert choose_search_grid(t([0, 200000]), 4, 3) == (4, 2)
     assert choose_search_grid(torch.from_numpy(cfg5_many_events_d8()["row_splits"]).long(), 8, 3) == (5, 1)
     assert choose_search_grid(t([0, 1000000]), 6, 3) == (5, 2)
     assert choose_search_grid(t([0, 6000, 10000]), 3, 3) == (3, 1)
