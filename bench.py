@@ -154,6 +154,14 @@ def main():
                 "kernel_ms": round(t_knn, 4),
                 # inputs + outputs of the timed launch: queries, int64 indices, distances, int32 sorted-space rows
                 "io_floor_bytes": 4.0 * D * n + 16.0 * K * n}
+    # what a plain device-to-device copy reaches on this box (1 GiB read + 1 GiB written), for orientation
+    del idx, dist, nbr_sorted
+    src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+    dst = torch.empty_like(src)
+    t_copy = float(np.median(timed(lambda: dst.copy_(src), 7)[2:]))
+    roofline["copy_gbs"] = round(2.0 * src.numel() * 4 / (t_copy * 1e-3) / 1e9, 1)
+    roofline["frac_of_copy"] = round(achieved / roofline["copy_gbs"], 4)
+    del src, dst
 
     result = {
         "metric": "kNN queries/sec and neighbours/sec at N=1M,D=3,K=64; % of HBM roofline",
