@@ -197,7 +197,7 @@ static int grad_table_size(int D)
 {
     int H = GRAD_H;
     const size_t d4 = (size_t)((D + 3) / 4);
-    while (H > 64 && 4 * (size_t)H * (4 + 16 * d4) > 49152) H >>= 1;
+    while (H > 64 && (size_t)H * (4 + 16 * d4) > 12288) H >>= 1;       // at most 12 KB per wavefront
     return H;
 }
 
@@ -244,7 +244,19 @@ __global__ __launch_bounds__(256) void k_sorted_points(const float *__restrict__
     xs[t] = make_float4(v[0], v[1], v[2], v[3]);
 }
 
-__global__ __launch_bounds__(256) void k_knn_grad_sorted(const float *__restrict__ gd, const int *__restrict__ nbr,
+#ifndef GSB
+#define GSB 1        // wavefronts per block of the sorted-space gradient kernel: no cooperation inside a block, and
+#endif               // single-wavefront blocks pack the LDS of a CU best (0.83 -> 0.78 ms at N=1M, D=3, K=64)
+#ifndef GSH
+#define GSH 512      // table slots per wavefront where an entry is 16 bytes (D <= 3)
+#endif
+#ifndef GSW
+#define GSW 32       // queries per wavefront where an entry is 16 bytes (0.78 -> 0.74 ms against 24)
+#endif
+// PACK (D <= 3): a table entry is one float4 (x, y, z, target) - value and key in one 16-byte LDS access, 8 KB of
+// table per wavefront.
+template <bool PACK>
+__global__ __launch_bounds__(64 * GSB) void k_knn_grad_sorted(const float *__restrict__ gd, const int *__restrict__ nbr,
                                                          const float4 *__restrict__ xs,
                                                          const uint32_t *__restrict__ order, float *__restrict__ gx,
                                                          int64_t n, int K, int D, int H, int *__restrict__ status)
@@ -253,25 +265,31 @@ __global__ __launch_bounds__(256) void k_knn_grad_sorted(const float *__restrict
     const int lane = fgc_lane();
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int D4 = (D + 3) >> 2;
-    const size_t wave_bytes = (size_t)H * (4 + 16 * (size_t)D4);
+    const size_t wave_bytes = PACK ? (size_t)H * 16 : (size_t)H * (4 + 16 * (size_t)D4);
     float4 *vals = (float4 *)(s_raw + wave_bytes * wv);
-    unsigned *keys = (unsigned *)(s_raw + wave_bytes * wv + (size_t)H * 16 * D4);
-    for (int t = lane; t < H; t += 64) keys[t] = GRAD_EMPTY;
-    for (int t = lane; t < H * D4; t += 64) vals[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+    unsigned *keys = PACK ? (unsigned *)vals + 3 : (unsigned *)(s_raw + wave_bytes * wv + (size_t)H * 16 * D4);
+    constexpr int KS = PACK ? 4 : 1;           // words between the keys of consecutive slots
+    constexpr int NQ = PACK ? GSW : GW;        // queries per wavefront
+    if (PACK) {
+        for (int t = lane; t < H; t += 64) vals[t] = make_float4(0.f, 0.f, 0.f, __uint_as_float(GRAD_EMPTY));
+    } else {
+        for (int t = lane; t < H; t += 64) keys[t] = GRAD_EMPTY;
+        for (int t = lane; t < H * D4; t += 64) vals[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     const unsigned hmask = (unsigned)H - 1u;
     bool bad = false;
     auto slot_of = [&](unsigned m) -> int {
         unsigned h = (m * 2654435761u) >> 7;
         for (int p = 0; p < GRAD_PROBES; p++) {
             const unsigned sl = (h + p) & hmask;
-            const unsigned old = atomicCAS(&keys[sl], GRAD_EMPTY, m);
+            const unsigned old = atomicCAS(&keys[sl * KS], GRAD_EMPTY, m);
             if (old == GRAD_EMPTY || old == m) return (int)sl;
         }
         return -1;
     };
 
-    const int64_t wave0 = ((int64_t)blockIdx.x * 4 + wv) * GW;
-    for (int q0 = 0; q0 < GW; q0 += GU) {
+    const int64_t wave0 = ((int64_t)blockIdx.x * GSB + wv) * NQ;
+    for (int q0 = 0; q0 < NQ; q0 += GU) {
         int64_t r[GU], qo[GU];
         bool qv[GU];
 #pragma unroll
@@ -312,7 +330,8 @@ __global__ __launch_bounds__(256) void k_knn_grad_sorted(const float *__restrict
                     self[3] = (c4 * 4 + 3 < D) ? fgc_wave_sum(add.w) : 0.f;
                     if (m[u] >= 0 && sl[u] >= 0) {
                         float4 v = vals[sl[u] * D4 + c4];
-                        v.x += add.x; v.y += add.y; v.z += add.z; v.w += add.w;
+                        v.x += add.x; v.y += add.y; v.z += add.z;
+                        if (!PACK) v.w += add.w;              // PACK: the fourth word is the key, written back as read
                         vals[sl[u] * D4 + c4] = v;
                     }
                     const bool ovf = m[u] >= 0 && sl[u] < 0;
@@ -325,7 +344,8 @@ __global__ __launch_bounds__(256) void k_knn_grad_sorted(const float *__restrict
                         if (lane == 0) {
                             if (ss >= 0) {
                                 float4 v = vals[ss * D4 + c4];
-                                v.x -= self[0]; v.y -= self[1]; v.z -= self[2]; v.w -= self[3];
+                                v.x -= self[0]; v.y -= self[1]; v.z -= self[2];
+                                if (!PACK) v.w -= self[3];
                                 vals[ss * D4 + c4] = v;
                             } else {
 #pragma unroll
@@ -341,7 +361,7 @@ __global__ __launch_bounds__(256) void k_knn_grad_sorted(const float *__restrict
     const float *vflat = (const float *)vals;
     for (int t = lane; t < H * D4 * 4; t += 64) {
         const int sl = t / (D4 * 4), c = t - sl * (D4 * 4);
-        const unsigned m = keys[sl];
+        const unsigned m = keys[sl * KS];
         if (m == GRAD_EMPTY || c >= D) continue;
         const float v = vflat[t];
         if (v != 0.f) atomicAdd(&gx[(int64_t)order[m] * D + c], v);
@@ -374,12 +394,19 @@ extern "C" int fgc_binned_select_knn_grad_sorted_f32(const float *d_grad_distsq,
     hipLaunchKernelGGL(k_sorted_points, dim3((unsigned)fgc_cdiv(n_vert * D4, 256)), dim3(256), 0, s, d_coords,
                        (const uint32_t *)d_order, n_vert, (int)n_coords, D4, xs);
     FGC_LAUNCH_CHECK();
-    const int H = grad_table_size(n_coords);
-    const size_t lds = 4 * (size_t)H * (4 + 16 * (size_t)D4);
-    const unsigned blocks = (unsigned)fgc_cdiv(n_vert, 4 * GW);
-    hipLaunchKernelGGL(k_knn_grad_sorted, dim3(blocks), dim3(256), lds, s, d_grad_distsq, d_nbr_sorted,
-                       (const float4 *)xs, (const uint32_t *)d_order, d_grad_coords, n_vert, (int)K, (int)n_coords, H,
-                       d_status);
+    if (n_coords <= 3) {
+        const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GSB * GSW);
+        hipLaunchKernelGGL((k_knn_grad_sorted<true>), dim3(blocks), dim3(64 * GSB), GSB * (size_t)GSH * 16, s,
+                           d_grad_distsq, d_nbr_sorted, (const float4 *)xs, (const uint32_t *)d_order, d_grad_coords,
+                           n_vert, (int)K, (int)n_coords, GSH, d_status);
+    } else {
+        const int H = grad_table_size(n_coords);
+        const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GSB * GW);
+        hipLaunchKernelGGL((k_knn_grad_sorted<false>), dim3(blocks), dim3(64 * GSB),
+                           GSB * (size_t)H * (4 + 16 * (size_t)D4), s, d_grad_distsq, d_nbr_sorted,
+                           (const float4 *)xs, (const uint32_t *)d_order, d_grad_coords, n_vert, (int)K,
+                           (int)n_coords, H, d_status);
+    }
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
