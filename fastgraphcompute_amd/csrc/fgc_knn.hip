@@ -412,9 +412,23 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                         } else flo = mid;
                     }
                 }
+                if (total <= K + slack || sel != 0xfffffffeu) {
+                    // the selected seeds fit the (still empty) pool as they are: one compaction over the registers
+                    int base = fgc_readlane_i(cnt, q);
 #pragma unroll
-                for (int s = 0; s < SMAX; s++)
-                    push(q, __uint_as_float(ds[s]), ((ra + s) << 6) + lane, ds[s] <= sel);
+                    for (int s = 0; s < SMAX; s++) {
+                        const bool want = ds[s] <= sel;
+                        const unsigned long long wm = fgc_ballot(want);
+                        if (want) pool[q * CAP + base + fgc_mbcnt(wm)] = make_uint2(ds[s], (unsigned)(((ra + s) << 6) + lane));
+                        base += __popcll(wm);
+                    }
+                    cnt = (lane == q) ? base : cnt;
+                } else {
+                    // no bound with K .. K + slack seeds below it (many equal distances): through the pool
+#pragma unroll
+                    for (int s = 0; s < SMAX; s++)
+                        push(q, __uint_as_float(ds[s]), ((ra + s) << 6) + lane, ds[s] <= sel);
+                }
             }
         }
 
