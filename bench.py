@@ -22,7 +22,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 # HBM bytes per k_knn launch at the default workload, from two rocprofv3 --pmc runs (FETCH_SIZE x 1.99 KiB
 # + WRITE_SIZE x 1.00 KiB, factors from a plain copy kernel in the same runs)
-KNN_TRAFFIC_CFG4_BYTES = 1282.8e6
+KNN_TRAFFIC_CFG4_BYTES = 1282.9e6
 
 
 def main():
