@@ -164,7 +164,9 @@ def main():
     del src, dst
 
     result = {
-        "metric": "kNN queries/sec and neighbours/sec at N=1M,D=3,K=64; % of HBM roofline",
+        "metric": ("kNN queries/sec and neighbours/sec at N=1M,D=3,K=64; % of HBM roofline"
+                   if (args.workload == "cfg4" and args.scale == 1.0) else
+                   "kNN queries/sec and neighbours/sec at N=%d,D=%d,K=%d; %% of HBM roofline" % (n, D, K)),
         "value": round(n / t_step, 1), "unit": "queries/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(t_step * 1e3, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
