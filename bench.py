@@ -398,6 +398,25 @@ def cpu_baseline(w, K, n, budget_s):
     nq3 = (n + stride3 - 1) // stride3
     many = {"value": round(nq3 / t3, 1), "unit": "queries/s", "cores": threads, "kind": "port",
             "sample": "every %d-th query (%d queries, %.1f s), OpenMP over queries" % (stride3, nq3, t3)}
+    # the reference's own compiled CPU kernel (oracle/_ref, when it was built) has no query stride, so it is timed
+    # on the same generator at a tenth of the points, next to the restatement on identical inputs: the ratio says
+    # how far the restatement's rate stands for the reference's
+    if O.ref_lib() is not None and w["name"].startswith("cfg4"):
+        from fastgraphcompute_amd import workloads
+        ws = workloads.CONFIGS["cfg4"](0.1)
+        ss = O.sorted_space(ws["coords"], ws["row_splits"], K)
+        sargs = (ss["scoords"], ss["sbin"], ss["sdbin"], ss["bin_boundaries"], ss["n_bins"], ss["bin_width"], K)
+        ns = ws["coords"].shape[0]
+        t0 = time.perf_counter()
+        ri, rd, _, _ = O.knn_sorted(*sargs, use_ref=True)
+        t_ref = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        pi, pd, _, _ = O.knn_sorted(*sargs, n_threads=1)
+        t_port = time.perf_counter() - t0
+        one["reference_check"] = {
+            "sample": "cfg4 generator at scale 0.1 (%d points), all queries, one core" % ns,
+            "reference_queries_per_s": round(ns / t_ref, 1), "port_queries_per_s": round(ns / t_port, 1),
+            "identical_results": bool((ri == pi).all() and (rd == pd).all())}
     return one, many
 
 
