@@ -375,10 +375,12 @@ __global__ __launch_bounds__(256) void k_bin_keys(const float *__restrict__ coor
 }
 
 // ---------------------------------------------------------------------------
-// LSD radix sort, 8-bit digits, stable.  Tile = 4 waves x 16 chunks x 64 keys.
+// LSD radix sort, 8-bit digits, stable.  Tile = 4 waves x CH chunks x 64 keys; the passes are short and bound by
+// latency, so small tiles (many blocks in flight) win: CH = 4 up to RS_SMALL_N keys, 8 beyond (1 M keys: 16 chunks
+// 0.209 ms for the whole preparation stage, 8 chunks 0.193, 4 chunks 0.202; 200 k keys: 0.124 / 0.094 / 0.082).
 // ---------------------------------------------------------------------------
-#define RS_TILE 4096
-#define RS_CHUNKS 16
+#define RS_MIN_TILE (256 * 4)
+#define RS_SMALL_N 700000
 
 // lanes of this wave holding the same digit (valid lanes only)
 __device__ __forceinline__ unsigned long long match_digit(int digit, bool valid)
@@ -393,9 +395,11 @@ __device__ __forceinline__ unsigned long long match_digit(int digit, bool valid)
 }
 
 // block_hist is digit-major: block_hist[digit * nblk + blk]
+template <int RS_CHUNKS>
 __global__ __launch_bounds__(256) void k_rs_hist(const uint32_t *__restrict__ keys, int n, int shift,
                                                  int nblk, uint32_t *__restrict__ block_hist)
 {
+    constexpr int RS_TILE = 256 * RS_CHUNKS;
     __shared__ uint32_t s_h[256];
     s_h[threadIdx.x] = 0;
     __syncthreads();
@@ -440,6 +444,7 @@ __global__ __launch_bounds__(256) void k_rs_scan_rows(uint32_t *__restrict__ blo
     if (t == 0) digit_total[blockIdx.x] = s_carry;
 }
 
+template <int RS_CHUNKS>
 __global__ __launch_bounds__(256) void k_rs_scatter(const uint32_t *__restrict__ keys_in,
                                                     const uint32_t *__restrict__ vals_in,
                                                     uint32_t *__restrict__ keys_out,
@@ -447,6 +452,7 @@ __global__ __launch_bounds__(256) void k_rs_scatter(const uint32_t *__restrict__
                                                     int nblk, const uint32_t *__restrict__ block_hist,
                                                     const uint32_t *__restrict__ digit_total)
 {
+    constexpr int RS_TILE = 256 * RS_CHUNKS;
     __shared__ uint32_t s_cnt[4][256];
     __shared__ uint32_t s_dig[256];   // exclusive scan of the digit totals
     {
@@ -522,7 +528,7 @@ __global__ __launch_bounds__(256) void k_rs_scatter(const uint32_t *__restrict__
 
 size_t fgc_sort_workspace_bytes(int64_t n)
 {
-    int64_t nblk = fgc_cdiv(n > 0 ? n : 1, RS_TILE);
+    int64_t nblk = fgc_cdiv(n > 0 ? n : 1, RS_MIN_TILE);   // the smallest tile has the most blocks
     return fgc_align((size_t)n * 4) * 2 /* ping-pong keys / vals */ + fgc_align((size_t)nblk * 256 * 4) +
            fgc_align(256 * 4) /* digit totals */;
 }
@@ -538,20 +544,26 @@ int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void 
     uint32_t *k_alt = (uint32_t *)w; w += fgc_align((size_t)n * 4);
     uint32_t *v_alt = (uint32_t *)w; w += fgc_align((size_t)n * 4);
     uint32_t *hist = (uint32_t *)w;
-    int nblk = (int)fgc_cdiv(n, RS_TILE);
-    uint32_t *digit_total = (uint32_t *)(w + fgc_align((size_t)nblk * 256 * 4));
-    if ((int64_t)nblk * 256 >= (1ll << 31)) return FGC_EINVAL;
+    const bool small = n <= RS_SMALL_N;
+    const int nblk = (int)fgc_cdiv(n, small ? 256 * 4 : 256 * 8);
+    uint32_t *digit_total = (uint32_t *)(w + fgc_align((size_t)fgc_cdiv(n > 0 ? n : 1, RS_MIN_TILE) * 256 * 4));
+    if ((int64_t)fgc_cdiv(n, RS_MIN_TILE) * 256 >= (1ll << 31)) return FGC_EINVAL;
     uint32_t *kin = keys, *vin = vals_given ? vals : nullptr, *kout = k_alt, *vout = v_alt;
     int passes = (key_bits + 7) / 8;
     if (passes < 1) passes = 1;
     for (int p = 0; p < passes; p++) {
         int shift = p * 8;
-        hipLaunchKernelGGL(k_rs_hist, dim3(nblk), dim3(256), 0, s, kin, (int)n, shift, nblk, hist);
+        if (small) hipLaunchKernelGGL(k_rs_hist<4>, dim3(nblk), dim3(256), 0, s, kin, (int)n, shift, nblk, hist);
+        else hipLaunchKernelGGL(k_rs_hist<8>, dim3(nblk), dim3(256), 0, s, kin, (int)n, shift, nblk, hist);
         FGC_LAUNCH_CHECK();
         hipLaunchKernelGGL(k_rs_scan_rows, dim3(256), dim3(256), 0, s, hist, nblk, digit_total);
         FGC_LAUNCH_CHECK();
-        hipLaunchKernelGGL(k_rs_scatter, dim3(nblk), dim3(256), 0, s, kin, vin, kout, vout, (int)n, shift,
-                           nblk, hist, digit_total);
+        if (small)
+            hipLaunchKernelGGL(k_rs_scatter<4>, dim3(nblk), dim3(256), 0, s, kin, vin, kout, vout, (int)n, shift,
+                               nblk, hist, digit_total);
+        else
+            hipLaunchKernelGGL(k_rs_scatter<8>, dim3(nblk), dim3(256), 0, s, kin, vin, kout, vout, (int)n, shift,
+                               nblk, hist, digit_total);
         FGC_LAUNCH_CHECK();
         kin = kout; vin = vout;
         if (kout == k_alt) { kout = keys; vout = vals; } else { kout = k_alt; vout = v_alt; }
