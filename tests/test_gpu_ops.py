@@ -78,7 +78,8 @@ def test_select_with_default(oracle):
 
 
 # ---------------------------------------------------------------- kNN gradient
-@pytest.mark.parametrize("n,D,K", [(1000, 2, 5), (1000, 4, 10), (3000, 3, 64), (2000, 8, 100), (500, 3, 200)])
+@pytest.mark.parametrize("n,D,K", [(1000, 2, 5), (1000, 4, 10), (3000, 3, 64), (2000, 8, 100), (500, 3, 200),
+                                    (1500, 6, 80), (1200, 10, 90)])
 def test_grad_vs_checker(oracle, n, D, K):
     from fastgraphcompute_amd.extensions import binned_select_knn_grad
     rng = np.random.default_rng(n + D + K)
@@ -129,6 +130,26 @@ def test_grad_reference_style_autograd(D, K):
     assert torch.equal(idx_s, i_ref)
     assert torch.allclose(dist_s, d_ref, atol=1e-5, rtol=1e-3)
     assert torch.allclose(g, g_ref, atol=1e-5, rtol=1e-3)
+
+
+@pytest.mark.parametrize("D,K", [(5, 40), (6, 70), (8, 100), (10, 90), (13, 64)])
+def test_grad_autograd_wide_points(D, K):
+    # points of five or more coordinates, where most (query, neighbour) pairs miss the on-chip tables and reach
+    # memory as 32-byte updates: the op's backward against autograd through the distances recomputed from the
+    # returned neighbour rows (independent of the order of nearly tied neighbours)
+    from fastgraphcompute_amd import binned_select_knn
+    torch.manual_seed(D * 100 + K)
+    n = 1500
+    coords = (torch.rand((n, D), dtype=torch.float32) - 0.5).cuda().requires_grad_(True)
+    rs = torch.tensor([0, 600, n], dtype=torch.int64, device="cuda")
+    offs = (torch.rand((n, K)) - 0.5).cuda()
+    idx, dist = binned_select_knn(K, coords, rs)
+    g = torch.autograd.grad(((dist + offs) ** 2).sum() - dist.sum(), coords)[0]
+    c64 = coords.detach().double().requires_grad_(True)
+    d_ref = ((c64[idx] - c64[:, None, :]) ** 2).sum(-1)
+    assert torch.allclose(dist.double(), d_ref, atol=1e-6, rtol=1e-5)
+    g_ref = torch.autograd.grad(((d_ref + offs.double()) ** 2).sum() - d_ref.sum(), c64)[0]
+    assert _rel_err(g.cpu().numpy(), g_ref.cpu().numpy()) < DIST_RTOL
 
 
 def test_grad_none_and_no_grad_inputs():
