@@ -115,3 +115,38 @@ def test_cfg3_gravnet_full(oracle):
     cm, cx, _ = oracle.gravnet_aggregate(ih, dh, prop.cpu().numpy())
     assert np.abs(fm.cpu().numpy() - cm).max() <= DIST_RTOL * np.abs(cm).max()
     assert np.abs(fx.cpu().numpy() - cx).max() <= DIST_RTOL * np.abs(cx).max()
+
+
+def test_more_than_2_31_output_entries():
+    """36 M points with K = 64: 2.3e9 entries per output array, past every 32-bit offset.  Sampled exhaustive
+    search on the device (first and last rows of each event included) and, for the gradient, translation
+    invariance: the coordinate gradients of all points sum to zero."""
+    from fastgraphcompute_amd import binned_select_knn
+    free, _ = torch.cuda.mem_get_info()
+    if free < 80 * 2 ** 30:
+        pytest.skip("needs about 60 GB of device memory")
+    n, K = 36_000_000, 64
+    torch.manual_seed(7)
+    coords = torch.rand((n, 3), device="cuda").requires_grad_(True)
+    cut = n // 3
+    rs = torch.tensor([0, cut, n], dtype=torch.int64, device="cuda")
+    idx, dist = binned_select_knn(K, coords, rs)
+    assert int((idx < 0).sum().item()) == 0
+    c = coords.detach()
+    g = torch.Generator().manual_seed(3)
+    sample = torch.cat([torch.tensor([0, 1, cut - 1, cut, n - 2, n - 1]), torch.randint(0, n, (58,), generator=g)])
+    for qi in sample.tolist():
+        lo, hi = (0, cut) if qi < cut else (cut, n)
+        d = ((c[lo:hi] - c[qi]) ** 2).sum(1)
+        ref_d = torch.sort(torch.topk(d, K, largest=False).values).values
+        got_d = torch.sort(dist[qi].detach()).values
+        assert torch.allclose(got_d, ref_d, rtol=DIST_RTOL, atol=1e-12), qi
+        row = idx[qi]
+        assert row[0].item() == qi and row.min().item() >= lo and row.max().item() < hi, qi
+        assert torch.allclose(((c[row] - c[qi]) ** 2).sum(1), dist[qi].detach(), rtol=DIST_RTOL, atol=1e-12), qi
+    del d
+    gd = torch.randn((n, K), device="cuda")
+    (dist * gd).sum().backward()
+    gr = coords.grad.double()
+    assert (gr.sum(0).abs() / gr.abs().sum(0)).max().item() < 1e-6
+    assert bool(coords.grad[-1000:].abs().sum(1).gt(0).all())
