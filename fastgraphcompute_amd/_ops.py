@@ -10,6 +10,7 @@ Two ops have no counterpart in the reference: the fused GravNet aggregation and
 the float32 select_with_default kernel.
 """
 import struct
+import threading
 import weakref
 from typing import List, Optional, Tuple
 
@@ -162,17 +163,21 @@ def knn_grad(grad_distsq: torch.Tensor, idx: torch.Tensor, coords: torch.Tensor,
     return out
 
 
-_PINNED = {}
+_PINNED = threading.local()
 
 
 def _pinned_status(dev: torch.device) -> torch.Tensor:
-    """One pinned int32[4] per device for the asynchronous read-back of the status word (each use ends with a
-    wait on its own event, so the buffer is free again when the next call starts)."""
+    """One pinned int32[4] per device and host thread for the asynchronous read-back of the status word (each use
+    ends with a wait on its own event, so the buffer is free again when the thread's next call starts; calls from
+    other threads have buffers of their own)."""
     key = dev.index if dev.index is not None else torch.cuda.current_device()
-    buf = _PINNED.get(key)
+    bufs = getattr(_PINNED, "bufs", None)
+    if bufs is None:
+        bufs = _PINNED.bufs = {}
+    buf = bufs.get(key)
     if buf is None:
         buf = torch.empty(4, dtype=torch.int32, pin_memory=True)
-        _PINNED[key] = buf
+        bufs[key] = buf
     return buf
 
 

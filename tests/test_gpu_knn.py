@@ -292,3 +292,55 @@ def test_row_splits_host_copy_follows_the_tensor(oracle):
     i4, d4 = binned_select_knn(8, c, rs)
     oi, od = oracle.binned_select_knn(8, coords, np.array([0, 500, 3000]))
     assert_knn_equal(i4.cpu().numpy(), d4.cpu().numpy(), oi, od, what="new tensor")
+
+
+def test_two_host_threads_on_their_own_streams():
+    """Calls from two host threads, each on a stream of its own, do not see each other's state: one thread searches
+    valid points over and over and must get the same rows as a call on its own, the other feeds non-finite
+    coordinates and must get the input error every time - and only that thread."""
+    import threading
+    from fastgraphcompute_amd import binned_select_knn
+    rng = np.random.default_rng(77)
+    good = torch.from_numpy(rng.random((60000, 3)).astype(np.float32)).cuda()
+    rs_good = torch.tensor([0, 25000, 60000], dtype=torch.int64, device="cuda")
+    bad_h = rng.random((40000, 3)).astype(np.float32)
+    bad_h[12345, 1] = np.nan
+    bad = torch.from_numpy(bad_h).cuda()
+    rs_bad = torch.tensor([0, 40000], dtype=torch.int64, device="cuda")
+    ref_i, ref_d = binned_select_knn(24, good, rs_good)
+    torch.cuda.synchronize()
+    out = {"good_ok": 0, "good_err": [], "bad_raised": 0, "bad_other": []}
+
+    def run_good():
+        s = torch.cuda.Stream()
+        with torch.cuda.stream(s):
+            for _ in range(25):
+                try:
+                    i, d = binned_select_knn(24, good, rs_good)
+                    s.synchronize()
+                    if torch.equal(i, ref_i) and torch.equal(d, ref_d):
+                        out["good_ok"] += 1
+                    else:
+                        out["good_err"].append("different rows")
+                except Exception as e:  # noqa: BLE001
+                    out["good_err"].append(repr(e))
+
+    def run_bad():
+        s = torch.cuda.Stream()
+        with torch.cuda.stream(s):
+            for _ in range(25):
+                try:
+                    binned_select_knn(24, bad, rs_bad)
+                    s.synchronize()
+                    out["bad_other"].append("no error")
+                except RuntimeError as e:
+                    if "non-finite" in str(e):
+                        out["bad_raised"] += 1
+                    else:
+                        out["bad_other"].append(repr(e))
+
+    ta, tb = threading.Thread(target=run_good), threading.Thread(target=run_bad)
+    ta.start(); tb.start(); ta.join(); tb.join()
+    torch.cuda.synchronize()
+    assert out["good_err"] == [] and out["good_ok"] == 25, out
+    assert out["bad_other"] == [] and out["bad_raised"] == 25, out
