@@ -385,7 +385,19 @@ def cpu_baseline(w, K, n, budget_s):
     _, _, ev2, _ = O.knn_sorted(*args, n_threads=1, query_stride=stride2)
     t = time.perf_counter() - t0
     nq = (n + stride2 - 1) // stride2
-    one = {"value": round(nq / t, 1), "unit": "queries/s", "cores": 1, "kind": "port",
+    cpu_model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for line in fh:
+                if line.startswith("model name"):
+                    cpu_model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    import torch
+    host = {"cpu_model": cpu_model, "nproc": os.cpu_count(), "usable_cores": len(os.sched_getaffinity(0)),
+            "torch_threads": torch.get_num_threads()}
+    one = {"value": round(nq / t, 1), "unit": "queries/s", "cores": 1, "kind": "port", "host": host,
            "sample": "every %d-th query of the bin-sorted workload (%d queries, %.1f s, %d distance "
                      "evaluations); kNN search kernel only, binning and sort excluded" % (stride2, nq, t, ev2)}
     # the same restatement with OpenMP over the queries on the cores this process may use (the reference's CPU
