@@ -28,14 +28,24 @@ Pinning status (what fixes each function independently of this restatement):
                                    test_binned_select_knn.py:209-226),
                                    oracle/_ref bit for bit.
   select_with_default,
-  gravnet_aggregate, gravnet_forward
-                                   restated with stock torch CPU ops exactly as
-                                   gnn_ops.py:79-109 composes them; the
-                                   reference's tests hold no numeric values for
-                                   GravNetOp (tests/test_gnn_ops.py checks
-                                   shapes and script-vs-eager only), so the C
-                                   aggregation kernel is pinned against that
-                                   torch composition and autograd.
+  gravnet_aggregate, gravnet_aggregate_torch, gravnet_forward_torch
+                                   the reference's tests hold no numeric values
+                                   for GravNetOp (tests/test_gnn_ops.py checks
+                                   shapes and script-vs-eager only), so these are
+                                   pinned by what gnn_ops.py:90-102 fixes
+                                   mathematically (tests/test_oracle_gravnet.py):
+                                   hand-computed known answers with weights 1,
+                                   1/2, 1/4 (padding counts as 0, the mean
+                                   divides by K, the padding's 0 can be the
+                                   maximum, the first of two equal maxima takes
+                                   the gradient; forward, both gradients, and the
+                                   whole layer with hand-set weights), closed
+                                   forms (zero distances = numpy.take + mean /
+                                   max, K = 1 = own features, a common distance
+                                   scales the result), a float64 loop over the
+                                   definition, and central differences of that
+                                   loop for the aggregation's and the layer's
+                                   gradients.
   oc_helper_inputs,
   max_same_valued_entries_per_row_split
                                    numpy.unique per row split, the routine the

@@ -45,6 +45,25 @@ def _sample_check(w, gi, gd, n_samples, seed):
     assert_knn_equal(gi[q], gd[q], bi, bd, "sampled exhaustive search")
 
 
+def _autograd_gradient_check(oracle, w, seed):
+    """The backward that binned_select_knn's autograd runs (the sorted-space gradient kernel, fed by the search's
+    own sorted neighbour rows) against the checker's gradient on the same neighbour rows, at full size."""
+    from fastgraphcompute_amd import binned_select_knn
+    coords = torch.from_numpy(w["coords"]).cuda().requires_grad_(True)
+    idx, dist = binned_select_knn(w["K"], coords, torch.from_numpy(w["row_splits"]).cuda())
+    up = w.get("grad_distsq")
+    if up is None:
+        up = np.random.default_rng(seed).standard_normal(tuple(dist.shape)).astype(np.float32)
+    dist.backward(torch.from_numpy(up).cuda())
+    got = coords.grad.cpu().numpy()
+    gi = idx.cpu().numpy()
+    exp = oracle.knn_grad(up, gi, w["coords"])
+    scale = np.abs(exp).max()
+    assert np.abs(got - exp).max() <= DIST_RTOL * scale
+    assert np.abs(got.astype(np.float64).sum(axis=0)).max() <= 1e-3 * scale
+    return gi, dist.detach().cpu().numpy()
+
+
 def test_cfg4_full_forward_and_gradient(oracle):
     from fastgraphcompute_amd.workloads import cfg4_zipf_blobs
     from fastgraphcompute_amd.extensions import binned_select_knn_grad
@@ -65,6 +84,10 @@ def test_cfg4_full_forward_and_gradient(oracle):
     scale = np.abs(exp).max()
     assert np.abs(got - exp).max() <= DIST_RTOL * scale
     assert np.abs(got.astype(np.float64).sum(axis=0)).max() <= 1e-3 * scale
+    # the backward the benchmark times: autograd through the whole call (sorted-space kernel, 16-byte entries)
+    ai, ad = _autograd_gradient_check(oracle, w, 0)
+    np.testing.assert_array_equal(ai, gi)
+    np.testing.assert_array_equal(ad, gd)
     # linearity in the upstream gradient
     g2 = torch.from_numpy(np.random.default_rng(5).standard_normal(g1.shape).astype(np.float32)).cuda()
     lin = binned_select_knn_grad(2.0 * g1 - 0.5 * g2, it, x).cpu().numpy()
@@ -79,6 +102,7 @@ def test_cfg2_full_against_checker(oracle):
     check_knn_properties(gi, gd, w["coords"], w["row_splits"], w["K"])
     oi, od = oracle.binned_select_knn(w["K"], w["coords"], w["row_splits"], n_threads=16)
     assert_knn_equal(gi, gd, oi, od)
+    _autograd_gradient_check(oracle, w, 12)      # D = 4: the wide-entry variant of the sorted-space kernel
 
 
 def test_cfg5_full_sampled(oracle):
@@ -87,6 +111,9 @@ def test_cfg5_full_sampled(oracle):
     gi, gd = _run(w)
     check_knn_properties(gi, gd, w["coords"], w["row_splits"], w["K"])
     _sample_check(w, gi, gd, 400, 6)
+    # D = 8, K = 100: the wide-entry gradient kernel where nearly every pair leaves the on-chip table
+    # (both overflow paths), against the checker on all 50 M pairs
+    _autograd_gradient_check(oracle, w, 15)
 
 
 def test_cfg3_gravnet_full(oracle):
@@ -115,6 +142,46 @@ def test_cfg3_gravnet_full(oracle):
     cm, cx, _ = oracle.gravnet_aggregate(ih, dh, prop.cpu().numpy())
     assert np.abs(fm.cpu().numpy() - cm).max() <= DIST_RTOL * np.abs(cm).max()
     assert np.abs(fx.cpu().numpy() - cx).max() <= DIST_RTOL * np.abs(cx).max()
+
+
+def test_cfg3_gravnet_backward_against_checker(oracle):
+    """x.grad and the parameter gradients of the cfg3 layer against autograd through the checker's CPU layer
+    (torch Linear, checker kNN and gradient, torch aggregation), on the first 2 x 12 000 points of the cfg3
+    input with the cfg3 weights.  The learned coordinates differ in the last bits between the GPU and CPU
+    products, so the comparison is at 2e-3 of each gradient's largest entry."""
+    from fastgraphcompute_amd.workloads import cfg3_gravnet
+    from fastgraphcompute_amd.gnn_ops import GravNetOp
+    w = cfg3_gravnet()
+    per = 12000
+    half = w["x"].shape[0] // 2
+    sel = np.concatenate([np.arange(per), half + np.arange(per)])
+    x_h = torch.from_numpy(w["x"][sel].copy())
+    g_h = torch.from_numpy(w["out_grad"][sel].copy())
+    rs = np.array([0, per, 2 * per], dtype=np.int32)
+    torch.manual_seed(w["weight_seed"])
+    op = GravNetOp(w["in_channels"], w["out_channels"], w["space_dimensions"], w["propagate_dimensions"], w["K"])
+    wt = {kk: v.detach().clone().requires_grad_(True) for kk, v in op.state_dict().items()}
+    xr = x_h.clone().requires_grad_(True)
+    out_r, idx_r, d_r, _ = oracle.gravnet_forward_torch(xr, rs, wt, w["K"], n_threads=16)
+    (out_r * g_h).sum().backward()
+    op = op.cuda()
+    xg = x_h.cuda().requires_grad_(True)
+    out, idx, dsq, _ = op(xg, torch.from_numpy(rs).cuda())
+    (out * g_h.cuda()).sum().backward()
+
+    def close(a, b, what, scale=None):
+        a, b = a.detach().cpu().double(), b.detach().double()
+        assert float((a - b).abs().max()) <= 2e-3 * (scale or float(b.abs().max())), what
+
+    close(out, out_r, "out")
+    close(torch.sort(dsq, 1).values, torch.sort(d_r, 1).values, "distsq")
+    close(xg.grad, xr.grad, "x.grad")
+    for name, p in op.named_parameters():
+        # a bias gradient is the plain sum of the rows whose products with x give the weight gradient; for the
+        # coordinate projection that sum is zero analytically (the distances do not change under a shift of
+        # all points), so it is compared on the scale of its layer's weight gradient
+        scale = float(wt[name.replace(".bias", ".weight")].grad.abs().max()) if name.endswith(".bias") else None
+        close(p.grad, wt[name].grad, name, scale)
 
 
 def test_more_than_2_31_output_entries():

@@ -232,3 +232,75 @@ def test_gravnet_op_shapes(C, P, k, S):
     assert set(op.state_dict().keys()) == {
         "space_transformations.weight", "space_transformations.bias", "propagate_transformations.weight",
         "propagate_transformations.bias", "output_transformations.0.weight", "output_transformations.0.bias"}
+
+
+# ---------------------------------------------------------------- hand-computed known answers (tests/golden)
+def _known():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "gravnet_known_answers.json")) as f:
+        return json.load(f)
+
+
+def test_gravnet_aggregate_known_answers():
+    # the HIP kernels on the hand-computed table the checker is pinned with (tests/test_oracle_gravnet.py):
+    # weights 1, 1/2, 1/4, padding counted as 0, mean over K, the padding's 0 as maximum, first of two equal maxima
+    import ctypes
+    from fastgraphcompute_amd import _lib
+    from fastgraphcompute_amd.gnn_ops import gravnet_aggregate
+    a = _known()["aggregate"]
+    idx = torch.tensor(a["idx"], device="cuda")
+    d = torch.tensor(a["distsq"], dtype=torch.float32, device="cuda", requires_grad=True)
+    f = torch.tensor(a["feat"], dtype=torch.float32, device="cuda", requires_grad=True)
+    fmean, fmax = gravnet_aggregate(idx, d, f)
+    np.testing.assert_allclose(fmean.detach().cpu().numpy(), a["fmean"], rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(fmax.detach().cpu().numpy(), a["fmax"], rtol=1e-6, atol=1e-7)
+    ((fmean * torch.tensor(a["grad_fmean"], device="cuda")).sum()
+     + (fmax * torch.tensor(a["grad_fmax"], device="cuda")).sum()).backward()
+    np.testing.assert_allclose(f.grad.cpu().numpy(), a["grad_feat"], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(d.grad.cpu().numpy(), a["grad_distsq"], rtol=1e-5, atol=1e-5)
+    # the arg-max slots, through the C ABI
+    n, K, P = 5, a["K"], a["P"]
+    m = torch.empty((n, P), device="cuda")
+    x = torch.empty((n, P), device="cuda")
+    am = torch.empty((n, P), dtype=torch.int32, device="cuda")
+    _lib.check(_lib.lib().fgc_gravnet_aggregate_fwd_f32(_lib.ptr(idx), _lib.ptr(d.detach()), _lib.ptr(f.detach()),
+                                                        _lib.ptr(m), _lib.ptr(x), _lib.ptr(am), n, K, P,
+                                                        _lib.stream_ptr()))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(am.cpu().numpy(), a["argmax"])
+
+
+def test_gravnet_layer_known_answers():
+    from fastgraphcompute_amd.gnn_ops import GravNetOp
+    from tests.test_oracle_gravnet import layer_weights
+    c = _known()["layer"]
+    op = GravNetOp(4, 8, 2, 2, c["k"])
+    op.load_state_dict(layer_weights())
+    op = op.cuda()
+    x = torch.tensor(c["x"], dtype=torch.float32, device="cuda")
+    out, idx, dsq, space = op(x, torch.tensor(c["row_splits"], device="cuda"))
+    idx, dsq = idx.cpu().numpy(), dsq.detach().cpu().numpy()
+    np.testing.assert_array_equal(idx[:, 0], np.arange(4))
+    np.testing.assert_array_equal(np.sort(idx, 1), np.sort(np.array(c["neighbour_sets"]), 1))
+    np.testing.assert_allclose(np.sort(dsq, 1), c["distsq_sorted"], rtol=1e-5, atol=1e-8)
+    expect = np.maximum(np.concatenate([np.array(c["x"]), np.array(c["fmean"]), np.array(c["fmax"])], 1), 0.0)
+    np.testing.assert_allclose(out.detach().cpu().numpy(), expect, rtol=1e-5, atol=1e-6)
+
+
+def test_gravnet_aggregate_closed_forms():
+    from fastgraphcompute_amd.gnn_ops import gravnet_aggregate
+    rng = np.random.default_rng(77)
+    n, K, P = 500, 9, 20
+    f = rng.standard_normal((n, P)).astype(np.float32)
+    idx = rng.integers(0, n, (n, K))
+    # all distances 0, no padding: numpy.take + mean / max
+    g = np.take(f, idx, axis=0)
+    m, x = gravnet_aggregate(torch.from_numpy(idx).cuda(), torch.zeros((n, K), device="cuda"), torch.from_numpy(f).cuda())
+    np.testing.assert_allclose(m.cpu().numpy(), g.mean(1), rtol=1e-6, atol=1e-6)
+    np.testing.assert_array_equal(x.cpu().numpy(), g.max(1))
+    # K = 1, self neighbour: own features
+    m, x = gravnet_aggregate(torch.arange(n, device="cuda")[:, None], torch.zeros((n, 1), device="cuda"),
+                             torch.from_numpy(f).cuda())
+    np.testing.assert_array_equal(m.cpu().numpy(), f)
+    np.testing.assert_array_equal(x.cpu().numpy(), f)
