@@ -26,6 +26,8 @@ SIGNATURES = {
     "fgc_binned_select_knn_workspace_bytes": (_sz, [_i64, _i32, _i32, c_i64p, _i32, _i32]),
     "fgc_binned_select_knn_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, c_i64p, _i32, _i32, _i32, c_i64p, _vp,
                                                  _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "fgc_binned_select_knn_noalloc_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, c_i64p, _i32, _i32, _i32, c_i64p, _vp,
+                                                         _i32, _vp, _vp, _vp, _vp]),
     "fgc_binned_knn_prepare_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, c_i64p, _i32, _i32, _i32, c_i64p, _vp, _vp,
                                                   _vp, _sz, _vp]),
     "fgc_binned_knn_search_f32": (ctypes.c_int, [_i64, _i32, c_i64p, _i32, _i32, _i32, c_i64p, _i32, _i32, _vp,

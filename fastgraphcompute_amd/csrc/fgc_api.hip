@@ -2,6 +2,7 @@
 #include "fgc_common.h"
 #include "fgc_internal.h"
 #include <cstdlib>
+#include <mutex>
 
 extern "C" int fgc_version(void) { return 100; }
 
@@ -12,6 +13,9 @@ extern "C" const char *fgc_error_string(int code)
     case FGC_EINVAL: return "invalid argument (shape, size or row splits)";
     case FGC_ENOSPACE: return "workspace too small";
     case FGC_EUNSUPPORTED: return "Unsupported number of binning dimensions.";
+    case FGC_ETOOLARGE:
+        return "input needs more scratch memory than the fixed area of the no-allocation entry point "
+               "(FGC_NOALLOC_SCRATCH_BYTES); use fgc_binned_select_knn_f32 with a workspace of the caller";
     default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -261,4 +265,57 @@ extern "C" int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, 
     return fgc_binned_knn_search_f32(n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins,
                                      d_direction != nullptr, tf_compat, d_idx, d_distsq, nullptr, d_stats, d_ws,
                                      ws_bytes, stream);
+}
+
+// ---------------------------------------------------------------------------
+// The whole forward for callers that cannot allocate (code under HIP graph capture, tight serving loops): the
+// workspace is a fixed array in the code object's own device memory.  Every GPU the library runs on holds one
+// copy of it at its own address until the process ends; that address is looked up once per device.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[FGC_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];    // device address of `scratch` on each device, 0 = not looked up yet
+
+// address of this device's copy of `scratch` (the array's name is only a host-side handle for the lookup)
+int scratch_address(void **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return FGC_EINVAL;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return FGC_EINVAL;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return FGC_OK;
+}
+}  // namespace
+
+extern "C" int fgc_binned_select_knn_noalloc_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
+                                                 const int64_t *d_row_splits, const int64_t *row_splits_host,
+                                                 int32_t n_rs, int32_t K, int32_t n_bin_dims,
+                                                 const int64_t *n_bins, const int64_t *d_direction,
+                                                 int32_t tf_compat, int64_t *d_idx, float *d_distsq,
+                                                 int32_t *d_status, void *stream)
+{
+    if (n_vert < 0 || n_coords < 1 || n_rs < 2 || !n_bins || n_bin_dims < 1 || n_bin_dims > FGC_MAX_BIN_DIMS)
+        return FGC_EINVAL;
+    const size_t need = n_vert > 0 ? plan(n_vert, n_coords, n_bin_dims, n_bins, n_rs, d_direction != nullptr).total : 0;
+    if (need > (size_t)FGC_NOALLOC_SCRATCH_BYTES) return FGC_ETOOLARGE;
+    void *ws = nullptr;
+    int rc = scratch_address(&ws);
+    if (rc) return rc;
+    // every stage writes what it later reads (the workspace of the other entry points is uninitialised memory
+    // too), so nothing of the previous call's contents has to be cleared
+    return fgc_binned_select_knn_f32(d_coords, n_vert, n_coords, d_row_splits, row_splits_host, n_rs, K, n_bin_dims,
+                                     n_bins, d_direction, tf_compat, d_idx, d_distsq, d_status, nullptr, ws,
+                                     (size_t)FGC_NOALLOC_SCRATCH_BYTES, stream);
 }

@@ -32,6 +32,7 @@ extern "C" {
 #define FGC_EINVAL (-1)      /* bad shape / unsupported size                  */
 #define FGC_ENOSPACE (-2)    /* workspace too small                           */
 #define FGC_EUNSUPPORTED (-3)/* e.g. number of binned dims outside 1..5       */
+#define FGC_ETOOLARGE (-4)   /* input exceeds the fixed scratch of a no-allocation entry point */
 
 #define FGC_MAX_BIN_DIMS 5
 #define FGC_MAX_K 256        /* neighbours per query the kNN kernel supports  */
@@ -126,6 +127,29 @@ int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_c
                               const int64_t *d_direction, int32_t tf_compat,
                               int64_t *d_idx, float *d_distsq, int32_t *d_status,
                               uint64_t *d_stats, void *d_ws, size_t ws_bytes, void *stream);
+
+/* The whole forward without a workspace argument and without any allocation.
+ * No counterpart in the reference (its forward allocates every intermediate
+ * with torch::empty, binned_knn_autograd_kernel.cpp:118-139); it is for the
+ * callers that cannot allocate device memory or size a workspace: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Same arguments and results as fgc_binned_select_knn_f32 (no d_stats); the
+ * intermediates live in a fixed array of FGC_NOALLOC_SCRATCH_BYTES bytes that
+ * is part of the library's device code, one copy per GPU, held until the
+ * process ends.  The call allocates and frees nothing.
+ *   - An input whose workspace (fgc_binned_select_knn_workspace_bytes) exceeds
+ *     FGC_NOALLOC_SCRATCH_BYTES is rejected with FGC_ETOOLARGE (about one
+ *     million points with three coordinates fit).
+ *   - All calls on one GPU share that GPU's array: calls that overlap on one
+ *     GPU (two streams, two host threads) race.  Calls on one stream are safe.
+ *   - The current device at the call must be the one the pointers belong to.
+ */
+#define FGC_NOALLOC_SCRATCH_BYTES (32u << 20)
+int fgc_binned_select_knn_noalloc_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
+                                      const int64_t *d_row_splits, const int64_t *row_splits_host,
+                                      int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
+                                      const int64_t *d_direction, int32_t tf_compat,
+                                      int64_t *d_idx, float *d_distsq, int32_t *d_status, void *stream);
 
 /* The same forward in two stages sharing one workspace, for callers that
  * search one prepared point set more than once or time the stages apart:
