@@ -130,3 +130,32 @@ def test_ops_are_registered_and_wrappers_script():
     # scripting compiles without a device
     sm = torch.jit.script(GravNetOp(8, 6, 3, 5, 4))
     assert "binned_select_knn_autograd" in str(sm.graph) or "binned_select_knn" in str(sm.code)
+
+
+def test_integration_shim_compiles_against_the_header():
+    """The reference-side binding documented in INTEGRATION.md (the C++ a maintainer would put behind
+    BinnedKNNAutograd and the *_cuda_fn symbols) is compiled, syntax only, against include/fgc_hip.h and the torch
+    headers: argument counts and types of every call must match the header."""
+    import shutil
+    import subprocess
+    import tempfile
+    import torch.utils.cpp_extension as ce
+    if shutil.which("g++") is None:
+        pytest.skip("no g++")
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    blocks = re.findall(r"```cpp\n(.*?)```", text, flags=re.S)
+    assert blocks, "INTEGRATION.md holds no C++ block"
+    src = "\n".join(blocks)
+    for fn in ("fgc_binned_select_knn_f32", "fgc_binned_select_knn_grad_f32", "fgc_index_replacer_i64",
+               "fgc_bin_points_f32"):
+        assert fn in src, fn
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "shim.cpp")
+        with open(path, "w") as f:
+            f.write(src)
+        cmd = ["g++", "-std=c++17", "-fsyntax-only", "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM",
+               "-I", os.path.join(ROOT, "include"), "-I", "/opt/rocm/include", "-I", "/usr/include/python3.10"]
+        for inc in ce.include_paths():
+            cmd += ["-I", inc]
+        r = subprocess.run(cmd + [path], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-4000:]
