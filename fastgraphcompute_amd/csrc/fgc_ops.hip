@@ -33,14 +33,14 @@ extern "C" int fgc_index_replacer_i64(const int64_t *d_in, const int64_t *d_repl
 // side then sees one 16-byte update per target instead of one per coordinate, and it is the number of such
 // updates that bounds the atomic rate.  Wave-uniform call (all lanes, same c0).
 __device__ __forceinline__ void grad_overflow_add(unsigned long long ovf_mask, bool ovf, int target, float4 add,
-                                                  int c0, int D, float *__restrict__ gx, int lane)
+                                                  int c0, int D, int ld, float *__restrict__ gx, int lane)
 {
     if (__popcll(ovf_mask) <= 6) {
         if (ovf) {
-            if (c0 + 0 < D) atomicAdd(&gx[(int64_t)target * D + c0 + 0], add.x);
-            if (c0 + 1 < D) atomicAdd(&gx[(int64_t)target * D + c0 + 1], add.y);
-            if (c0 + 2 < D) atomicAdd(&gx[(int64_t)target * D + c0 + 2], add.z);
-            if (c0 + 3 < D) atomicAdd(&gx[(int64_t)target * D + c0 + 3], add.w);
+            if (c0 + 0 < D) atomicAdd(&gx[(int64_t)target * ld + c0 + 0], add.x);
+            if (c0 + 1 < D) atomicAdd(&gx[(int64_t)target * ld + c0 + 1], add.y);
+            if (c0 + 2 < D) atomicAdd(&gx[(int64_t)target * ld + c0 + 2], add.z);
+            if (c0 + 3 < D) atomicAdd(&gx[(int64_t)target * ld + c0 + 3], add.w);
         }
         return;
     }
@@ -54,7 +54,7 @@ __device__ __forceinline__ void grad_overflow_add(unsigned long long ovf_mask, b
         const float v0 = __shfl(add.x, e, 64), v1 = __shfl(add.y, e, 64);
         const float v2 = __shfl(add.z, e, 64), v3 = __shfl(add.w, e, 64);
         const float v = comp == 0 ? v0 : comp == 1 ? v1 : comp == 2 ? v2 : v3;
-        if (te >= 0 && c0 + comp < D) atomicAdd(&gx[(int64_t)te * D + c0 + comp], v);
+        if (te >= 0 && c0 + comp < D) atomicAdd(&gx[(int64_t)te * ld + c0 + comp], v);
     }
 }
 
@@ -63,14 +63,14 @@ __device__ __forceinline__ void grad_overflow_add(unsigned long long ovf_mask, b
 // update per target instead of two 16-byte ones (N=500 k, D=8, K=100, where nearly every pair overflows: 3.6 ms
 // with one group per update).  Wave-uniform call.
 __device__ __forceinline__ void grad_overflow_add8(unsigned long long ovf_mask, bool ovf, int target, float4 lo,
-                                                   float4 hi, int c0, int D, float *__restrict__ gx, int lane)
+                                                   float4 hi, int c0, int D, int ld, float *__restrict__ gx, int lane)
 {
     if (__popcll(ovf_mask) <= 3) {
         if (ovf) {
             const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
             for (int e = 0; e < 8; e++)
-                if (c0 + e < D) atomicAdd(&gx[(int64_t)target * D + c0 + e], v[e]);
+                if (c0 + e < D) atomicAdd(&gx[(int64_t)target * ld + c0 + e], v[e]);
         }
         return;
     }
@@ -86,7 +86,7 @@ __device__ __forceinline__ void grad_overflow_add8(unsigned long long ovf_mask, 
         const float va = (comp & 2) ? ((comp & 1) ? v3 : v2) : ((comp & 1) ? v1 : v0);
         const float vb = (comp & 2) ? ((comp & 1) ? v7 : v6) : ((comp & 1) ? v5 : v4);
         const float v = (comp & 4) ? vb : va;
-        if (te >= 0 && c0 + comp < D) atomicAdd(&gx[(int64_t)te * D + c0 + comp], v);
+        if (te >= 0 && c0 + comp < D) atomicAdd(&gx[(int64_t)te * ld + c0 + comp], v);
     }
 }
 
@@ -98,13 +98,14 @@ __device__ __forceinline__ void grad_overflow_add8(unsigned long long ovf_mask, 
 // in the bin-sorted order when `order` is given, so their neighbourhoods
 // overlap - lane k owning neighbour slot k, and first combines all contributions
 // to the same target point in its own LDS hash table (open addressing).  The
-// neighbours of one query are distinct points, so the lanes of one instruction
-// never update the same table entry and, the table being private to the
-// wavefront, the update is a plain LDS read-add-write of one float4 - no float
-// atomics on chip.  Only the distinct targets of the wavefront go to global
-// memory, one float atomic per coordinate with a target's coordinates in
-// adjacent lanes.  Pairs that find no table slot within a few probes go to
-// global memory directly.
+// table is private to the wavefront and within one instruction every slot is
+// updated by one lane only, so the update is a plain LDS read-add-write of one
+// float4 - no float atomics on chip.  The neighbours of one query are normally
+// distinct points; a row that names a point twice is legal input, and the lanes
+// that then share a slot are told apart through an owner byte (see below).
+// Only the distinct targets of the wavefront go to global memory, one float
+// atomic per coordinate with a target's coordinates in adjacent lanes.  Pairs
+// that find no table slot within a few probes go to global memory directly.
 #ifndef GW
 #define GW 24          // queries per wavefront
 #endif
@@ -126,9 +127,10 @@ __global__ __launch_bounds__(256) void k_knn_grad(const float *__restrict__ gd, 
     const int lane = fgc_lane();
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // uniform by construction
     const int D4 = (D + 3) >> 2;                       // float4 groups per point
-    const size_t wave_bytes = (size_t)H * (4 + 16 * (size_t)D4);
+    const size_t wave_bytes = (size_t)H * (8 + 16 * (size_t)D4);
     float4 *vals = (float4 *)(s_raw + wave_bytes * wv);                  // [H][D4]
     unsigned *keys = (unsigned *)(s_raw + wave_bytes * wv + (size_t)H * 16 * D4);   // [H]
+    unsigned char *owner = s_raw + wave_bytes * wv + (size_t)H * (16 * (size_t)D4 + 4);   // [H]
     for (int t = lane; t < H; t += 64) keys[t] = GRAD_EMPTY;
     for (int t = lane; t < H * D4; t += 64) vals[t] = make_float4(0.f, 0.f, 0.f, 0.f);
     const unsigned hmask = (unsigned)H - 1u;
@@ -169,6 +171,13 @@ __global__ __launch_bounds__(256) void k_knn_grad(const float *__restrict__ gd, 
             for (int u = 0; u < GU; u++) {
                 if (m[u] >= n) { bad = true; m[u] = -1; }
                 sl[u] = (m[u] >= 0) ? slot_of((unsigned)m[u]) : -1;
+                // a row may name the same point twice (any index tensor can be passed to this op): the lanes that
+                // share a slot in this instruction write their number into the slot's owner byte, the one that
+                // reads its own number back updates the table, the others add to memory directly
+                if (sl[u] >= 0) owner[sl[u]] = (unsigned char)lane;
+                asm volatile("" ::: "memory");             // the byte is read back from LDS, not from the register
+                if (sl[u] >= 0 && owner[sl[u]] != (unsigned char)lane) sl[u] = -1;
+                asm volatile("" ::: "memory");
             }
             float4 addp[GU];       // the even float4 group of an overflowing pair, until its partner is known
 #pragma unroll
@@ -185,7 +194,7 @@ __global__ __launch_bounds__(256) void k_knn_grad(const float *__restrict__ gd, 
                         self[e] = (c < D) ? fgc_wave_sum(add[e]) : 0.f;
                     }
                     if (m[u] >= 0 && sl[u] >= 0) {
-                        // distinct targets within the instruction, private table: plain read-add-write
+                        // one lane per slot within the instruction, private table: plain read-add-write
                         float4 v = vals[sl[u] * D4 + c4];
                         v.x += add[0]; v.y += add[1]; v.z += add[2]; v.w += add[3];
                         vals[sl[u] * D4 + c4] = v;
@@ -196,8 +205,8 @@ __global__ __launch_bounds__(256) void k_knn_grad(const float *__restrict__ gd, 
                         // float4 groups leave in pairs (one 32-byte update per target), an unpaired last one alone
                         const float4 a4 = make_float4(add[0], add[1], add[2], add[3]);
                         if (!(c4 & 1) && c4 + 1 < D4) addp[u] = a4;
-                        else if (c4 & 1) grad_overflow_add8(om, ovf, (int)m[u], addp[u], a4, (c4 - 1) * 4, D, gx, lane);
-                        else grad_overflow_add(om, ovf, (int)m[u], a4, c4 * 4, D, gx, lane);
+                        else if (c4 & 1) grad_overflow_add8(om, ovf, (int)m[u], addp[u], a4, (c4 - 1) * 4, D, D, gx, lane);
+                        else grad_overflow_add(om, ovf, (int)m[u], a4, c4 * 4, D, D, gx, lane);
                     }
                     // the query's own share, after the neighbours' updates of this instruction
                     if (qv[u]) {
@@ -236,7 +245,7 @@ static int grad_table_size(int D)
 {
     int H = GRAD_H;
     const size_t d4 = (size_t)((D + 3) / 4);
-    while (H > 64 && (size_t)H * (4 + 16 * d4) > 12288) H >>= 1;       // at most 12 KB per wavefront
+    while (H > 64 && (size_t)H * (8 + 16 * d4) > 12288) H >>= 1;       // at most 12 KB per wavefront
     return H;
 }
 
@@ -252,7 +261,7 @@ extern "C" int fgc_binned_select_knn_grad_f32(const float *d_grad_distsq, const 
     int rc = fgc_fill_u32(d_grad_coords, 0u, n_vert * n_coords, s);
     if (rc) return rc;
     const int H = grad_table_size(n_coords);
-    const size_t lds = 4 * (size_t)H * (4 + 16 * (size_t)((n_coords + 3) / 4));
+    const size_t lds = 4 * (size_t)H * (8 + 16 * (size_t)((n_coords + 3) / 4));
     const unsigned blocks = (unsigned)fgc_cdiv(n_vert, 4 * GW);
     hipLaunchKernelGGL(k_knn_grad, dim3(blocks), dim3(256), lds, s, d_grad_distsq, d_idx, d_coords,
                        d_grad_coords, (const uint32_t *)d_order, n_vert, (int)K, (int)n_coords, H, d_status);
@@ -283,144 +292,254 @@ __global__ __launch_bounds__(256) void k_sorted_points(const float *__restrict__
     xs[t] = make_float4(v[0], v[1], v[2], v[3]);
 }
 
-#ifndef GSB
-#define GSB 1        // wavefronts per block of the sorted-space gradient kernel: no cooperation inside a block, and
-#endif               // single-wavefront blocks pack the LDS of a CU best (0.83 -> 0.78 ms at N=1M, D=3, K=64)
 #ifndef GSH
 #define GSH 512      // table slots per wavefront where an entry is 16 bytes (D <= 3)
 #endif
 #ifndef GSW
-#define GSW 32       // queries per wavefront where an entry is 16 bytes (0.78 -> 0.74 ms against 24)
+#define GSW 32       // queries per wavefront where an entry is 16 bytes
 #endif
-// PACK (D <= 3): a table entry is one float4 (x, y, z, target) - value and key in one 16-byte LDS access, 8 KB of
-// table per wavefront.
+
+// Totals of 16 per-lane values over the 64 lanes, in 36 instead of 16 x 11 instructions: each exchange step
+// halves the number of values a lane still carries (the lane keeps the half its own bit selects and hands the
+// other half to its partner).  Returns, in every lane L, the total of value number L >> 2.
+__device__ __forceinline__ float fgc_wave_reduce16(const float (&v)[16], int lane)
+{
+    float a[8], b[4], c[2];
+#pragma unroll
+    for (int t = 0; t < 8; t++) {      // partner lane ^ 32: lower half keeps values 0..7, upper half 8..15
+        const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[t]), __float_as_uint(v[t + 8]), false, false);
+        a[t] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {      // partner lane ^ 16: even rows keep t, odd rows t + 4
+        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a[t]), __float_as_uint(a[t + 4]), false, false);
+        b[t] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
+    const bool b3 = (lane & 8) != 0, b2 = (lane & 4) != 0;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {      // partner lane ^ 8
+        const float keep = b3 ? b[t + 2] : b[t], send = b3 ? b[t] : b[t + 2];
+        c[t] = keep + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send), 0x128, 0xf, 0xf, true));
+    }
+    const float keep = b2 ? c[1] : c[0], send = b2 ? c[0] : c[1];
+    float z = keep;
+    {                                   // partner lane ^ 4 = mirror the half row (^7), then reverse the quad (^3)
+        const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(send), 0x141, 0xf, 0xf, true);
+        z += __int_as_float(__builtin_amdgcn_update_dpp(0, t, 0x1B, 0xf, 0xf, true));
+    }
+    z += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(z), 0x4E, 0xf, 0xf, true));   // ^ 2
+    z += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(z), 0xB1, 0xf, 0xf, true));   // ^ 1
+    return z;
+}
+
+#ifndef GRAD_OWNER_T
+#define GRAD_OWNER_T unsigned char
+#endif
+
+// A wavefront (= one block: nothing is shared inside a block, and small blocks pack the LDS of a CU best) takes NQ
+// consecutive rows of the sorted order, four at a time, lane k owning neighbour slot k, and combines the
+// contributions per target in a two-way LDS table: the first slot of target m is m mod H.  Targets are sorted
+// positions and the neighbours of consecutive rows are mostly positions close by, which this mapping sends to
+// distinct slots - the table is a dense window around the tile that wraps around for the far targets; a target
+// whose first slot holds another point tries a second one, shifted by a hash of m / H (so a far run of
+// consecutive positions stays a run of consecutive slots).  Who may use a slot is settled per instruction without
+// compare-and-swap loops: every lane writes its lane number into the slot's owner cell and reads it back; the
+// lane that finds its own number owns the slot for this instruction and may use it if the slot's tag is its
+// target (or the slot is empty: it takes it).  Everybody else - the loser of a collision, a second lane with the
+// same target (repeated index in a row), a target whose slots both hold other points - sends its contribution to
+// memory directly.  So the update of a table entry is a plain LDS read-add-write that no two lanes of an
+// instruction share.  The rows' own shares (-sum over the slots) are summed for four rows and four coordinates
+// at once (fgc_wave_reduce16) and go to slots taken for the tile's own rows up front.
+// Loads run two steps ahead of the arithmetic: while step s is combined on chip, the neighbour coordinates of
+// step s + 1 are being gathered and the index / upstream-gradient rows of step s + 2 are on their way.
+// The gradient is accumulated in the sorted order too (gxs, rows of D4 * 4 floats): the tables are flushed with
+// the coordinates of a target in adjacent lanes and neighbouring targets in neighbouring lanes, which for the
+// window part are neighbouring addresses; k_unsort_grad moves the rows to the original order.
+// PACK (D <= 3): a table entry is one float4 (x, y, z, tag) - value and tag in one 16-byte LDS access.
 template <bool PACK>
-__global__ __launch_bounds__(64 * GSB) void k_knn_grad_sorted(const float *__restrict__ gd, const int *__restrict__ nbr,
-                                                         const float4 *__restrict__ xs,
-                                                         const uint32_t *__restrict__ order, float *__restrict__ gx,
-                                                         int64_t n, int K, int D, int H, int *__restrict__ status)
+__global__ __launch_bounds__(64) void k_knn_grad_sorted(const float *__restrict__ gd, const int *__restrict__ nbr,
+                                                        const float4 *__restrict__ xs,
+                                                        const uint32_t *__restrict__ order, float *__restrict__ gxs,
+                                                        int64_t n, int K, int D, int H, int *__restrict__ status)
 {
     extern __shared__ __align__(16) unsigned char s_raw[];
     const int lane = fgc_lane();
-    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int D4 = (D + 3) >> 2;
-    const size_t wave_bytes = PACK ? (size_t)H * 16 : (size_t)H * (4 + 16 * (size_t)D4);
-    float4 *vals = (float4 *)(s_raw + wave_bytes * wv);
-    unsigned *keys = PACK ? (unsigned *)vals + 3 : (unsigned *)(s_raw + wave_bytes * wv + (size_t)H * 16 * D4);
-    constexpr int KS = PACK ? 4 : 1;           // words between the keys of consecutive slots
-    constexpr int NQ = PACK ? GSW : GW;        // queries per wavefront
+    const int D4 = PACK ? 1 : (D + 3) >> 2;
+    const int ld = D4 * 4;                     // floats per row of xs and gxs
+    float4 *vals = (float4 *)s_raw;            // [H][D4]
+    unsigned *tags = PACK ? (unsigned *)vals + 3 : (unsigned *)(s_raw + (size_t)H * 16 * D4);
+    GRAD_OWNER_T *owner = (GRAD_OWNER_T *)(s_raw + (PACK ? (size_t)H * 16 : (size_t)H * (16 * (size_t)D4 + 4)));
+    constexpr int KS = PACK ? 4 : 1;           // words between the tags of consecutive slots
+    constexpr int NQ = PACK ? GSW : GW;        // rows per wavefront
+    static_assert(GU == 4 && NQ % GU == 0 && NQ <= 64, "fgc_wave_reduce16 sums four rows of four coordinates");
     if (PACK) {
         for (int t = lane; t < H; t += 64) vals[t] = make_float4(0.f, 0.f, 0.f, __uint_as_float(GRAD_EMPTY));
     } else {
-        for (int t = lane; t < H; t += 64) keys[t] = GRAD_EMPTY;
+        for (int t = lane; t < H; t += 64) tags[t] = GRAD_EMPTY;
         for (int t = lane; t < H * D4; t += 64) vals[t] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
     const unsigned hmask = (unsigned)H - 1u;
+    const int hbits = 31 - __builtin_clz((unsigned)H);
+    const int64_t wave0 = (int64_t)blockIdx.x * NQ;
+    // slots of the tile's own rows (consecutive positions: distinct slots); lane q keeps row q's original index
+    unsigned my_order = 0u;
+    if (lane < NQ && wave0 + lane < n) {
+        tags[(((unsigned)(wave0 + lane)) & hmask) * KS] = (unsigned)(wave0 + lane);
+        my_order = order[wave0 + lane];
+    }
+    const int *__restrict__ nb0 = nbr + wave0 * K;           // the tile's neighbour rows
     bool bad = false;
-    auto slot_of = [&](unsigned m) -> int {
-        unsigned h = (m * 2654435761u) >> 7;
-        for (int p = 0; p < GRAD_PROBES; p++) {
-            const unsigned sl = (h + p) & hmask;
-            const unsigned old = atomicCAS(&keys[sl * KS], GRAD_EMPTY, m);
-            if (old == GRAD_EMPTY || old == m) return (int)sl;
-        }
-        return -1;
-    };
+#ifdef FGC_GRAD_COUNTERS
+    unsigned n_pairs = 0, n_ovf = 0;
+#endif
 
-    const int64_t wave0 = ((int64_t)blockIdx.x * GSB + wv) * NQ;
-    for (int q0 = 0; q0 < NQ; q0 += GU) {
-        int64_t r[GU], qo[GU];
-        bool qv[GU];
+    // stage A of a step (rows q .. q + 3, slots k0 .. k0 + 63): neighbour positions and upstream gradients
+    auto stage_a = [&](int q, int k0, int (&m)[GU], float (&g)[GU]) {
+        const int k = k0 + lane;
 #pragma unroll
         for (int u = 0; u < GU; u++) {
-            r[u] = wave0 + q0 + u;
-            qv[u] = r[u] < n;
-            if (!qv[u]) r[u] = 0;
-            qo[u] = order[r[u]];
+            m[u] = -1; g[u] = 0.f;
+            if (q + u < NQ && wave0 + q + u < n && k < K) {
+                m[u] = nb0[(q + u) * K + k];
+                g[u] = gd[(int64_t)fgc_readlane_i((int)my_order, q + u) * K + k];
+            }
         }
-        for (int k0 = 0; k0 < K; k0 += 64) {
-            const int k = k0 + lane;
-            int m[GU], sl[GU];
-            float g[GU];
+    };
+    // stage B: the neighbours' coordinates (first float4 group)
+    auto stage_b = [&](int (&m)[GU], float4 (&x)[GU]) {
+#pragma unroll
+        for (int u = 0; u < GU; u++) {
+            if (m[u] >= n) { bad = true; m[u] = -1; }
+            x[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (m[u] >= 0) x[u] = xs[(int64_t)m[u] * D4];
+        }
+    };
+    // may this lane use slot s for target mm in this instruction?
+    auto try_slot = [&](bool want, unsigned s, unsigned mm) -> bool {
+        const unsigned tag = want ? tags[s * KS] : 0u;
+        if (want) owner[s] = (GRAD_OWNER_T)lane;
+        asm volatile("" ::: "memory");                     // the cell is read back from LDS, not from the register
+        const bool win = want && owner[s] == (GRAD_OWNER_T)lane;
+        const bool ok = win && (tag == mm || tag == GRAD_EMPTY);
+        if (ok && tag == GRAD_EMPTY) tags[s * KS] = mm;
+        asm volatile("" ::: "memory");
+        return ok;
+    };
+
+    int m1[GU], m2[GU];
+    float g1[GU], g2[GU];
+    float4 x1[GU];
+    int qa = 0, ka = 0;                        // step whose stage A is issued next
+    auto next_step = [&](int &q, int &k0) { k0 += 64; if (k0 >= K) { k0 = 0; q += GU; } };
+    stage_a(qa, ka, m1, g1); next_step(qa, ka);
+    stage_b(m1, x1);
+    stage_a(qa, ka, m2, g2); next_step(qa, ka);
+    int qc = 0, kc = 0;                        // step being combined
+    while (qc < NQ) {
+        int m[GU];
+        float g[GU];
+        float4 xm[GU];
+#pragma unroll
+        for (int u = 0; u < GU; u++) { m[u] = m1[u]; g[u] = g1[u]; xm[u] = x1[u]; m1[u] = m2[u]; g1[u] = g2[u]; }
+        stage_b(m1, x1);
+        stage_a(qa, ka, m2, g2); next_step(qa, ka);
+
+        int sl[GU];
+#pragma unroll
+        for (int u = 0; u < GU; u++) {
+            const bool valid = m[u] >= 0;
+            const unsigned mm = (unsigned)m[u];
+            const unsigned s1 = mm & hmask;
+            bool ok = try_slot(valid, s1, mm);
+            unsigned s = s1;
+            const bool again = valid && !ok;
+            if (fgc_ballot(again)) {
+                // an odd shift: never the first slot again (its owner of this instruction may be a lane with
+                // the same target)
+                const unsigned s2 = (s1 + ((((mm >> hbits) * 2654435761u) >> 20) | 1u)) & hmask;
+                const bool ok2 = try_slot(again, s2, mm);
+                if (again) { ok = ok2; s = s2; }
+            }
+            sl[u] = ok ? (int)s : -1;
+#ifdef FGC_GRAD_COUNTERS
+            n_pairs += (unsigned)__popcll(fgc_ballot(valid));
+            n_ovf += (unsigned)__popcll(fgc_ballot(valid && !ok));
+#endif
+        }
+        float4 addp[GU];       // the even float4 group of an overflowing pair, until its partner is known
+#pragma unroll
+        for (int u = 0; u < GU; u++) addp[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int c4 = 0; c4 < D4; c4++) {
+            float red[16];
 #pragma unroll
             for (int u = 0; u < GU; u++) {
-                m[u] = -1; g[u] = 0.f;
-                if (k < K && qv[u]) { m[u] = nbr[r[u] * K + k]; g[u] = gd[qo[u] * K + k]; }
-            }
-#pragma unroll
-            for (int u = 0; u < GU; u++) {
-                if (m[u] >= n) { bad = true; m[u] = -1; }
-                sl[u] = (m[u] >= 0) ? slot_of((unsigned)m[u]) : -1;
-            }
-            float4 addp[GU];       // the even float4 group of an overflowing pair, until its partner is known
-#pragma unroll
-            for (int u = 0; u < GU; u++) addp[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-            for (int c4 = 0; c4 < D4; c4++) {
-#pragma unroll
-                for (int u = 0; u < GU; u++) {
-                    const float4 xi = xs[r[u] * D4 + c4];
-                    float4 add = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (m[u] >= 0) {
-                        const float4 xm = xs[(int64_t)m[u] * D4 + c4];
-                        const float g2 = 2.f * g[u];
-                        add = make_float4(g2 * (xm.x - xi.x), g2 * (xm.y - xi.y), g2 * (xm.z - xi.z), g2 * (xm.w - xi.w));
-                    }
-                    float self[4];
-                    self[0] = fgc_wave_sum(add.x);
-                    self[1] = (c4 * 4 + 1 < D) ? fgc_wave_sum(add.y) : 0.f;
-                    self[2] = (c4 * 4 + 2 < D) ? fgc_wave_sum(add.z) : 0.f;
-                    self[3] = (c4 * 4 + 3 < D) ? fgc_wave_sum(add.w) : 0.f;
-                    if (m[u] >= 0 && sl[u] >= 0) {
-                        float4 v = vals[sl[u] * D4 + c4];
-                        v.x += add.x; v.y += add.y; v.z += add.z;
-                        if (!PACK) v.w += add.w;              // PACK: the fourth word is the key, written back as read
-                        vals[sl[u] * D4 + c4] = v;
-                    }
-                    const bool ovf = m[u] >= 0 && sl[u] < 0;
-                    const unsigned long long om = fgc_ballot(ovf);
-                    if (om) {
-                        // float4 groups leave in pairs (one 32-byte update per target), an unpaired last one alone
-                        if (!(c4 & 1) && c4 + 1 < D4) addp[u] = add;
-                        else if (c4 & 1)
-                            grad_overflow_add8(om, ovf, ovf ? (int)order[m[u]] : -1, addp[u], add, (c4 - 1) * 4, D, gx, lane);
-                        else grad_overflow_add(om, ovf, ovf ? (int)order[m[u]] : -1, add, c4 * 4, D, gx, lane);
-                    }
-                    if (qv[u]) {
-                        int ss = -1;
-                        if (lane == 0) ss = slot_of((unsigned)r[u]);
-                        ss = fgc_readlane_i(ss, 0);
-                        if (lane == 0) {
-                            if (ss >= 0) {
-                                float4 v = vals[ss * D4 + c4];
-                                v.x -= self[0]; v.y -= self[1]; v.z -= self[2];
-                                if (!PACK) v.w -= self[3];
-                                vals[ss * D4 + c4] = v;
-                            } else {
-#pragma unroll
-                                for (int e = 0; e < 4; e++)
-                                    if (c4 * 4 + e < D) atomicAdd(&gx[qo[u] * D + c4 * 4 + e], -self[e]);
-                            }
-                        }
-                    }
+                const int64_t row = (wave0 + qc + u < n) ? wave0 + qc + u : 0;
+                const float4 xi = xs[row * D4 + c4];
+                float4 add = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (m[u] >= 0) {
+                    const float4 xn = (PACK || c4 == 0) ? xm[u] : xs[(int64_t)m[u] * D4 + c4];
+                    const float gg = 2.f * g[u];
+                    add = make_float4(gg * (xn.x - xi.x), gg * (xn.y - xi.y), gg * (xn.z - xi.z), gg * (xn.w - xi.w));
+                }
+                red[u * 4 + 0] = add.x; red[u * 4 + 1] = add.y; red[u * 4 + 2] = add.z; red[u * 4 + 3] = add.w;
+                if (sl[u] >= 0) {
+                    float4 v = vals[sl[u] * D4 + c4];
+                    v.x += add.x; v.y += add.y; v.z += add.z;
+                    if (!PACK) v.w += add.w;              // PACK: the fourth word is the tag, written back as read
+                    vals[sl[u] * D4 + c4] = v;
+                }
+                const bool ovf = m[u] >= 0 && sl[u] < 0;
+                const unsigned long long om = fgc_ballot(ovf);
+                if (om) {
+                    // float4 groups leave in pairs (one 32-byte update per target), an unpaired last one alone
+                    if (!PACK && !(c4 & 1) && c4 + 1 < D4) addp[u] = add;
+                    else if (!PACK && (c4 & 1)) grad_overflow_add8(om, ovf, m[u], addp[u], add, (c4 - 1) * 4, D, ld, gxs, lane);
+                    else grad_overflow_add(om, ovf, m[u], add, c4 * 4, D, ld, gxs, lane);
                 }
             }
+            // the rows' own shares: lane L holds the total of row L >> 4, coordinate c4 * 4 + ((L >> 2) & 3)
+            const float tot = fgc_wave_reduce16(red, lane);
+            const int su = lane >> 4, se = (lane >> 2) & 3;
+            const int64_t sr = wave0 + qc + su;
+            if ((lane & 3) == 0 && sr < n && c4 * 4 + se < D) {
+                float *p = (float *)vals + ((size_t)(((unsigned)sr) & hmask) * D4 + c4) * 4 + se;
+                *p -= tot;
+            }
         }
+        next_step(qc, kc);
     }
+    // flush: one lane per (slot, coordinate); for the window part of the table neighbouring lanes hold
+    // neighbouring addresses
     const float *vflat = (const float *)vals;
-    for (int t = lane; t < H * D4 * 4; t += 64) {
-        const int sl = t / (D4 * 4), c = t - sl * (D4 * 4);
-        const unsigned m = keys[sl * KS];
+    for (int t = lane; t < H * ld; t += 64) {
+        const int sl = t / ld, c = t - sl * ld;
+        const unsigned m = tags[sl * KS];
         if (m == GRAD_EMPTY || c >= D) continue;
         const float v = vflat[t];
-        if (v != 0.f) atomicAdd(&gx[(int64_t)order[m] * D + c], v);
+        if (v != 0.f) atomicAdd(&gxs[(int64_t)m * ld + c], v);
     }
     if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
+#ifdef FGC_GRAD_COUNTERS
+    if (status && lane == 0) { atomicAdd(&status[2], (int)(n_pairs >> 6)); atomicAdd(&status[3], (int)(n_ovf >> 6)); }
+#endif
+}
+
+// rows of the sorted-space gradient to the original order: gx[order[r], :] = gxs[r, :D]
+__global__ __launch_bounds__(256) void k_unsort_grad(const float *__restrict__ gxs, const uint32_t *__restrict__ order,
+                                                     int64_t n, int D, int ld, float *__restrict__ gx)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n * ld) return;
+    const int64_t r = t / ld;
+    const int c = (int)(t - r * ld);
+    if (c < D) gx[(int64_t)order[r] * D + c] = gxs[t];
 }
 
 extern "C" size_t fgc_binned_select_knn_grad_sorted_workspace_bytes(int64_t n_vert, int32_t n_coords)
 {
     if (n_vert < 0 || n_coords < 1) return 0;
-    return fgc_align((size_t)(n_vert > 0 ? n_vert : 1) * (size_t)((n_coords + 3) / 4) * 16);
+    // the sorted copy of the points and the gradient in sorted order, both padded to whole float4 groups
+    return 2 * fgc_align((size_t)(n_vert > 0 ? n_vert : 1) * (size_t)((n_coords + 3) / 4) * 16);
 }
 
 extern "C" int fgc_binned_select_knn_grad_sorted_f32(const float *d_grad_distsq, const int32_t *d_nbr_sorted,
@@ -435,26 +554,30 @@ extern "C" int fgc_binned_select_knn_grad_sorted_f32(const float *d_grad_distsq,
     if (!d_grad_distsq || !d_nbr_sorted || !d_coords || !d_order || !d_grad_coords) return FGC_EINVAL;
     if (!d_ws || ws_bytes < fgc_binned_select_knn_grad_sorted_workspace_bytes(n_vert, n_coords)) return FGC_ENOSPACE;
     hipStream_t s = (hipStream_t)stream;
-    int rc = fgc_fill_u32(d_grad_coords, 0u, n_vert * n_coords, s);
-    if (rc) return rc;
     const int D4 = (n_coords + 3) / 4;
+    const size_t half = fgc_align((size_t)n_vert * D4 * 16);
     float4 *xs = (float4 *)d_ws;
+    float *gxs = (float *)((char *)d_ws + half);
+    int rc = fgc_fill_u32(gxs, 0u, n_vert * D4 * 4, s);
+    if (rc) return rc;
     hipLaunchKernelGGL(k_sorted_points, dim3((unsigned)fgc_cdiv(n_vert * D4, 256)), dim3(256), 0, s, d_coords,
                        (const uint32_t *)d_order, n_vert, (int)n_coords, D4, xs);
     FGC_LAUNCH_CHECK();
     if (n_coords <= 3) {
-        const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GSB * GSW);
-        hipLaunchKernelGGL((k_knn_grad_sorted<true>), dim3(blocks), dim3(64 * GSB), GSB * (size_t)GSH * 16, s,
-                           d_grad_distsq, d_nbr_sorted, (const float4 *)xs, (const uint32_t *)d_order, d_grad_coords,
-                           n_vert, (int)K, (int)n_coords, GSH, d_status);
+        const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GSW);
+        hipLaunchKernelGGL((k_knn_grad_sorted<true>), dim3(blocks), dim3(64), (size_t)GSH * (16 + sizeof(GRAD_OWNER_T)), s, d_grad_distsq,
+                           d_nbr_sorted, (const float4 *)xs, (const uint32_t *)d_order, gxs, n_vert, (int)K,
+                           (int)n_coords, GSH, d_status);
     } else {
         const int H = grad_table_size(n_coords);
-        const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GSB * GW);
-        hipLaunchKernelGGL((k_knn_grad_sorted<false>), dim3(blocks), dim3(64 * GSB),
-                           GSB * (size_t)H * (4 + 16 * (size_t)D4), s, d_grad_distsq, d_nbr_sorted,
-                           (const float4 *)xs, (const uint32_t *)d_order, d_grad_coords, n_vert, (int)K,
-                           (int)n_coords, H, d_status);
+        const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GW);
+        hipLaunchKernelGGL((k_knn_grad_sorted<false>), dim3(blocks), dim3(64), (size_t)H * (8 + 16 * (size_t)D4), s,
+                           d_grad_distsq, d_nbr_sorted, (const float4 *)xs, (const uint32_t *)d_order, gxs, n_vert,
+                           (int)K, (int)n_coords, H, d_status);
     }
+    FGC_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_unsort_grad, dim3((unsigned)fgc_cdiv(n_vert * D4 * 4, 256)), dim3(256), 0, s, gxs,
+                       (const uint32_t *)d_order, n_vert, (int)n_coords, D4 * 4, d_grad_coords);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }

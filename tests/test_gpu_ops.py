@@ -107,6 +107,48 @@ def test_grad_vs_checker(oracle, n, D, K):
     assert _rel_err(got, ref) < DIST_RTOL
 
 
+@pytest.mark.parametrize("D,K", [(3, 64), (2, 17), (8, 100), (5, 130)])
+def test_grad_rows_with_repeated_indices(oracle, D, K):
+    """Any index tensor may be handed to the gradient op: rows that name the same point several times (also the
+    query itself, also a whole row of one point) must accumulate every contribution, as the reference's sequential
+    loop does (binned_select_knn_grad_cpu.cpp:63-92).  Both kernels: the op in the original order and, through the
+    C ABI, the sorted-space kernel on rows with repeats."""
+    from fastgraphcompute_amd import _lib
+    from fastgraphcompute_amd.extensions import binned_select_knn_grad
+    rng = np.random.default_rng(D * 1000 + K)
+    n = 3000
+    coords = rng.random((n, D)).astype(np.float32)
+    idx = rng.integers(0, n, (n, K))
+    idx[:, 0] = np.arange(n)
+    idx[rng.random((n, K)) < 0.1] = -1
+    idx[:, 5] = idx[:, 3]                       # every row repeats a neighbour
+    idx[::3, 7:12] = idx[::3, 6:7]              # runs of one point
+    idx[5] = 17                                 # a whole row of one point
+    idx[6] = 6                                  # a whole row of the query itself
+    near = (np.arange(n)[:, None] + rng.integers(-40, 40, (n, K))) % n
+    idx[1000:2000] = np.where(idx[1000:2000] >= 0, near[1000:2000], -1)     # local rows: heavy sharing between rows
+    idx[1000:2000, 9] = idx[1000:2000, 2]
+    gd = rng.standard_normal((n, K)).astype(np.float32)
+    exp = oracle.knn_grad(gd, idx, coords)
+    x, g, it = torch.from_numpy(coords).cuda(), torch.from_numpy(gd).cuda(), torch.from_numpy(idx).cuda()
+    got = binned_select_knn_grad(g, it, x).cpu().numpy()
+    assert _rel_err(got, exp) < DIST_RTOL
+    # the sorted-space kernel with the identity as its order: rows and entries are then original indices
+    L = _lib.lib()
+    order = torch.arange(n, dtype=torch.int32, device="cuda")
+    nbr = it.to(torch.int32).contiguous()
+    out = torch.empty((n, D), device="cuda")
+    status = torch.zeros(4, dtype=torch.int32, device="cuda")
+    ws_bytes = L.fgc_binned_select_knn_grad_sorted_workspace_bytes(n, D)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    _lib.check(L.fgc_binned_select_knn_grad_sorted_f32(_lib.ptr(g), _lib.ptr(nbr), _lib.ptr(x), _lib.ptr(order),
+                                                       _lib.ptr(out), n, K, D, _lib.ptr(status), _lib.ptr(ws), ws_bytes,
+                                                       _lib.stream_ptr()))
+    torch.cuda.synchronize()
+    assert _rel_err(out.cpu().numpy(), exp) < DIST_RTOL
+    assert int(status[0].item()) == 0
+
+
 @pytest.mark.parametrize("D,K", [(2, 50), (4, 10)])
 def test_grad_reference_style_autograd(D, K):
     # tests/test_binned_select_knn.py:184-226 of the reference: gradient of a non-trivial loss through the op
