@@ -28,22 +28,14 @@ extern "C" int fgc_index_replacer_i64(const int64_t *d_in, const int64_t *d_repl
 }
 
 // Overflow of the per-wavefront table: the lanes flagged `ovf` add their float4 `add` to the four coordinates
-// c0 .. c0 + 3 of row `target` of gx.  With more than a few such lanes the values are exchanged between the lanes
-// so that each atomic instruction carries 16 targets with their four coordinates in adjacent lanes: the memory
-// side then sees one 16-byte update per target instead of one per coordinate, and it is the number of such
-// updates that bounds the atomic rate.  Wave-uniform call (all lanes, same c0).
+// c0 .. c0 + 3 of row `target` of gx (row stride ld).  The values are exchanged between the lanes so that each
+// atomic instruction carries 16 targets with their four coordinates in adjacent lanes: the memory side then sees
+// one 16-byte update per target instead of one per coordinate, and it is the number of such updates that bounds
+// the atomic rate (also with only a few lanes flagged: N=1M, D=3, K=64 0.54 -> 0.47 ms against issuing them from
+// the flagged lanes directly).  Wave-uniform call (all lanes, same c0).
 __device__ __forceinline__ void grad_overflow_add(unsigned long long ovf_mask, bool ovf, int target, float4 add,
                                                   int c0, int D, int ld, float *__restrict__ gx, int lane)
 {
-    if (__popcll(ovf_mask) <= 6) {
-        if (ovf) {
-            if (c0 + 0 < D) atomicAdd(&gx[(int64_t)target * ld + c0 + 0], add.x);
-            if (c0 + 1 < D) atomicAdd(&gx[(int64_t)target * ld + c0 + 1], add.y);
-            if (c0 + 2 < D) atomicAdd(&gx[(int64_t)target * ld + c0 + 2], add.z);
-            if (c0 + 3 < D) atomicAdd(&gx[(int64_t)target * ld + c0 + 3], add.w);
-        }
-        return;
-    }
     const int tgt = ovf ? target : -1;
     const int comp = lane & 3;
 #pragma unroll
@@ -279,17 +271,20 @@ extern "C" int fgc_binned_select_knn_grad_f32(const float *d_grad_distsq, const 
 // order (one 16-byte gather per neighbour and four coordinates), and only the upstream gradient row and the
 // final atomics go through the permutation.
 __global__ __launch_bounds__(256) void k_sorted_points(const float *__restrict__ x, const uint32_t *__restrict__ order,
-                                                       int64_t n, int D, int D4, float4 *__restrict__ xs)
+                                                       int64_t n, int D, int D4, float4 *__restrict__ xs,
+                                                       float4 *__restrict__ gxs)
 {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n * D4) return;
-    const int64_t r = t / D4;
-    const int c4 = (int)(t - r * D4);
+    int64_t r = t;
+    int c4 = 0;
+    if (D4 > 1) { r = t / D4; c4 = (int)(t - r * D4); }
     const int64_t o = order[r];
     float v[4];
 #pragma unroll
     for (int e = 0; e < 4; e++) v[e] = (c4 * 4 + e < D) ? x[o * D + c4 * 4 + e] : 0.f;
     xs[t] = make_float4(v[0], v[1], v[2], v[3]);
+    gxs[t] = make_float4(0.f, 0.f, 0.f, 0.f);       // the gradient accumulator in the same order starts at zero
 }
 
 #ifndef GSH
@@ -389,6 +384,7 @@ __global__ __launch_bounds__(64) void k_knn_grad_sorted(const float *__restrict_
     }
     const int *__restrict__ nb0 = nbr + wave0 * K;           // the tile's neighbour rows
     bool bad = false;
+
 #ifdef FGC_GRAD_COUNTERS
     unsigned n_pairs = 0, n_ovf = 0;
 #endif
@@ -489,7 +485,11 @@ __global__ __launch_bounds__(64) void k_knn_grad_sorted(const float *__restrict_
                     vals[sl[u] * D4 + c4] = v;
                 }
                 const bool ovf = m[u] >= 0 && sl[u] < 0;
+#ifndef GRAD_ABL_NOOVF
                 const unsigned long long om = fgc_ballot(ovf);
+#else
+                const unsigned long long om = fgc_ballot(ovf && add.x == 123.456f);
+#endif
                 if (om) {
                     // float4 groups leave in pairs (one 32-byte update per target), an unpaired last one alone
                     if (!PACK && !(c4 & 1) && c4 + 1 < D4) addp[u] = add;
@@ -516,7 +516,11 @@ __global__ __launch_bounds__(64) void k_knn_grad_sorted(const float *__restrict_
         const unsigned m = tags[sl * KS];
         if (m == GRAD_EMPTY || c >= D) continue;
         const float v = vflat[t];
+#ifndef GRAD_ABL_NOFLUSH
         if (v != 0.f) atomicAdd(&gxs[(int64_t)m * ld + c], v);
+#else
+        if (v == 123.456f) atomicAdd(&gxs[(int64_t)m * ld + c], v);
+#endif
     }
     if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
 #ifdef FGC_GRAD_COUNTERS
@@ -524,15 +528,21 @@ __global__ __launch_bounds__(64) void k_knn_grad_sorted(const float *__restrict_
 #endif
 }
 
-// rows of the sorted-space gradient to the original order: gx[order[r], :] = gxs[r, :D]
-__global__ __launch_bounds__(256) void k_unsort_grad(const float *__restrict__ gxs, const uint32_t *__restrict__ order,
-                                                     int64_t n, int D, int ld, float *__restrict__ gx)
+// rows of the sorted-space gradient to the original order: gx[order[r], :] = gxs[r, :D]; one thread per float4 group
+__global__ __launch_bounds__(256) void k_unsort_grad(const float4 *__restrict__ gxs, const uint32_t *__restrict__ order,
+                                                     int64_t n, int D, int D4, float *__restrict__ gx)
 {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= n * ld) return;
-    const int64_t r = t / ld;
-    const int c = (int)(t - r * ld);
-    if (c < D) gx[(int64_t)order[r] * D + c] = gxs[t];
+    if (t >= n * D4) return;
+    int64_t r = t;
+    int c4 = 0;
+    if (D4 > 1) { r = t / D4; c4 = (int)(t - r * D4); }
+    const float4 v = gxs[t];
+    float *dst = gx + (int64_t)order[r] * D + c4 * 4;
+    dst[0] = v.x;
+    if (c4 * 4 + 1 < D) dst[1] = v.y;
+    if (c4 * 4 + 2 < D) dst[2] = v.z;
+    if (c4 * 4 + 3 < D) dst[3] = v.w;
 }
 
 extern "C" size_t fgc_binned_select_knn_grad_sorted_workspace_bytes(int64_t n_vert, int32_t n_coords)
@@ -558,10 +568,8 @@ extern "C" int fgc_binned_select_knn_grad_sorted_f32(const float *d_grad_distsq,
     const size_t half = fgc_align((size_t)n_vert * D4 * 16);
     float4 *xs = (float4 *)d_ws;
     float *gxs = (float *)((char *)d_ws + half);
-    int rc = fgc_fill_u32(gxs, 0u, n_vert * D4 * 4, s);
-    if (rc) return rc;
     hipLaunchKernelGGL(k_sorted_points, dim3((unsigned)fgc_cdiv(n_vert * D4, 256)), dim3(256), 0, s, d_coords,
-                       (const uint32_t *)d_order, n_vert, (int)n_coords, D4, xs);
+                       (const uint32_t *)d_order, n_vert, (int)n_coords, D4, xs, (float4 *)gxs);
     FGC_LAUNCH_CHECK();
     if (n_coords <= 3) {
         const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GSW);
@@ -576,8 +584,8 @@ extern "C" int fgc_binned_select_knn_grad_sorted_f32(const float *d_grad_distsq,
                            (int)K, (int)n_coords, H, d_status);
     }
     FGC_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_unsort_grad, dim3((unsigned)fgc_cdiv(n_vert * D4 * 4, 256)), dim3(256), 0, s, gxs,
-                       (const uint32_t *)d_order, n_vert, (int)n_coords, D4 * 4, d_grad_coords);
+    hipLaunchKernelGGL(k_unsort_grad, dim3((unsigned)fgc_cdiv(n_vert * D4, 256)), dim3(256), 0, s, (const float4 *)gxs,
+                       (const uint32_t *)d_order, n_vert, (int)n_coords, D4, d_grad_coords);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
