@@ -20,9 +20,58 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
-# HBM bytes per k_knn launch at the default workload, from two rocprofv3 --pmc runs (FETCH_SIZE x 1.99 KiB
-# + WRITE_SIZE x 1.00 KiB, factors from a plain copy kernel in the same runs)
-KNN_TRAFFIC_CFG4_BYTES = 1282.9e6
+N_SIMD = 1024           # 256 compute units x 4 SIMDs; a VALU wavefront instruction occupies its SIMD for 4 cycles
+
+
+def profile_facts():
+    """Per-kernel figures that only a profiler run gives (HBM bytes per launch from FETCH_SIZE / WRITE_SIZE,
+    VALU wavefront instructions per launch), read from the `#bench-fact` lines of the committed rocprofv3 summaries
+    under profiles/: {(kernel, workload): {key: value, "file": name}}.  Both are properties of the kernel and the
+    input, not of the run, so they are combined here with the kernel time measured live."""
+    facts = {}
+    pdir = os.path.join(ROOT, "profiles")
+    if not os.path.isdir(pdir):
+        return facts
+    for name in sorted(os.listdir(pdir)):
+        if not name.endswith(".txt"):
+            continue
+        with open(os.path.join(pdir, name)) as fh:
+            for line in fh:
+                if not line.startswith("#bench-fact"):
+                    continue
+                kv = dict(tok.split("=", 1) for tok in line.split()[1:] if "=" in tok)
+                key = (kv.pop("kernel", ""), kv.pop("workload", ""))
+                ent = facts.setdefault(key, {"files": []})
+                for k, v in kv.items():
+                    ent[k] = float(v)
+                ent["files"].append("profiles/" + name)
+    return facts
+
+
+def roofline_entry(kernel, workload, alg_bytes, kernel_ms, clock_hz, useful_valu_insts=None, facts=None):
+    """The roofline object of one kernel: `achieved` / `frac` on ALGORITHMIC bytes (what a kernel without reuse
+    would have to move), and beside them what the hardware counters say: physical HBM traffic and its share of the
+    peak, and the share of the kernel's duration its SIMDs spend issuing VALU instructions."""
+    achieved = alg_bytes / (kernel_ms * 1e-3) / 1e9
+    r = {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+         "frac": round(achieved / HBM_PEAK_GBS, 4),
+         "frac_kind": "effective: algorithmic bytes / measured kernel time (reads served from registers, LDS and L2 "
+                      "count as if they came from memory; it can exceed the physical share, and 1)",
+         "algorithmic_bytes": alg_bytes, "kernel_ms": round(kernel_ms, 4), "traffic": None, "physical_gbs": None,
+         "physical_frac": None, "valu_issue_frac": None, "useful_valu_frac": None, "profile": None}
+    f = (facts or {}).get((kernel, workload))
+    if f:
+        r["profile"] = sorted(set(f["files"]))
+        if "traffic_bytes" in f:
+            r["traffic"] = f["traffic_bytes"]
+            r["physical_gbs"] = round(f["traffic_bytes"] / (kernel_ms * 1e-3) / 1e9, 1)
+            r["physical_frac"] = round(r["physical_gbs"] / HBM_PEAK_GBS, 4)
+        if "valu_wave_insts" in f:
+            r["valu_issue_frac"] = round(f["valu_wave_insts"] * 4.0 / (N_SIMD * kernel_ms * 1e-3 * clock_hz), 4)
+            if useful_valu_insts is not None:
+                r["useful_valu_frac"] = round(useful_valu_insts / f["valu_wave_insts"], 4)
+            r["binding_resource"] = "valu_issue" if r["valu_issue_frac"] >= 0.6 else "latency / atomic-update rate"
+    return r
 
 
 def main():
@@ -34,6 +83,9 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seconds", type=float, default=15.0)
+    ap.add_argument("--cpu-reference-full", action="store_true",
+                    help="also time the reference's own compiled CPU kernel (oracle/_ref) on ALL queries of the "
+                         "workload, one core; minutes at the default workload")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no multi-GPU part); "
@@ -145,15 +197,20 @@ def main():
 
     # algorithmic bytes of one search launch: every distance evaluation reads one
     # D-float candidate, every query is read once, every (idx, distsq) slot written once
+    facts = profile_facts() if args.scale == 1.0 else {}
+    clock_hz = torch.cuda.get_device_properties(dev).clock_rate * 1e3
     bytes_alg = 4.0 * D * c_eval + 4.0 * D * n + 12.0 * K * n
-    achieved = bytes_alg / (t_knn * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": "k_knn", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": KNN_TRAFFIC_CFG4_BYTES if (args.workload == "cfg4" and args.scale == 1.0) else None,
-                "algorithmic_bytes": bytes_alg, "distance_evaluations": c_eval,
-                "kernel_ms": round(t_knn, 4),
-                # inputs + outputs of the timed launch: queries, int64 indices, distances, int32 sorted-space rows
-                "io_floor_bytes": 4.0 * D * n + 16.0 * K * n}
+    # VALU wavefront instructions that are distance arithmetic: per 64 evaluations D subtractions, D
+    # multiplications, D - 1 additions, the compare, and the D + 1 broadcasts of the query and its bound
+    roofline = roofline_entry("k_knn", w["name"], bytes_alg, t_knn, clock_hz, (c_eval / 64.0) * (4 * D + 1), facts)
+    achieved = roofline["achieved"]
+    roofline["distance_evaluations"] = c_eval
+    # inputs + outputs of the timed launch: queries, int64 indices, distances, int32 sorted-space rows
+    roofline["io_floor_bytes"] = 4.0 * D * n + 16.0 * K * n
+    # gradient kernel: upstream gradient + neighbour rows + one D-float gather per pair + coordinates in, gradient out
+    grad_alg = 4.0 * K * n + 8.0 * K * n + 4.0 * D * n * K + 8.0 * D * n
+    roofline_grad = roofline_entry("k_knn_grad_sorted", w["name"], grad_alg, t_grad, clock_hz, None, facts)
+    roofline_grad["kernel_ms_includes"] = "sorted copy of the points, the gradient kernel, un-sort of the result"
     # what a plain device-to-device copy reaches on this box (1 GiB read + 1 GiB written), for orientation
     del idx, dist, nbr_sorted
     src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
@@ -179,10 +236,13 @@ def main():
                       "gradient": round(t_grad, 4)},
         "search_counters": {"distance_evaluations": c_eval, "candidate_chunks": chunks, "pool_prunes": inserts},
         "roofline": roofline,
+        "roofline_gradient": roofline_grad,
     }
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"], result["cpu_baseline_allcores"] = cpu_baseline(w, K, n, args.cpu_sample_seconds)
+    if args.cpu_reference_full:
+        result["cpu_baseline_reference_full"] = cpu_reference_full(w, K, n)
     print(json.dumps(result), flush=True)
 
 
@@ -364,6 +424,23 @@ def oc_helper_workload(args, dev):
                                   "kind": "port", "sample": "calc_m restatement on %d of %d objects (%.2f s per pass, 3 passes), "
                                   "object analysis excluded" % (sel.size, uv.size, tc)}
     print(json.dumps(result), flush=True)
+
+
+def cpu_reference_full(w, K, n):
+    """The reference's own CPU kernel (its sources compiled unmodified into oracle/_ref) on every query of the
+    workload, single-threaded as it is written (binned_select_knn_cpu.cpp:56-208 has no parallel loop), with the
+    reference's own grid (calculate_optimal_bins).  Search kernel only, like cpu_baseline."""
+    from oracle import oracle as O
+    if O.ref_lib() is None:
+        return {"value": None, "kind": "reference", "sample": "oracle/_ref is not built on this machine"}
+    s = O.sorted_space(w["coords"], w["row_splits"], K)
+    a = (s["scoords"], s["sbin"], s["sdbin"], s["bin_boundaries"], s["n_bins"], s["bin_width"], K)
+    t0 = time.perf_counter()
+    O.knn_sorted(*a, use_ref=True)
+    t = time.perf_counter() - t0
+    return {"value": round(n / t, 1), "unit": "queries/s", "cores": 1, "kind": "reference",
+            "sample": "all %d queries of the bin-sorted workload, %.1f s, n_bins %s; kNN search kernel only"
+                      % (n, t, [int(v) for v in s["n_bins"]])}
 
 
 def cpu_baseline(w, K, n, budget_s):

@@ -9,6 +9,7 @@ with `torch.library`; the implementations call libfgc_hip.so through ctypes.
 Two ops have no counterpart in the reference: the fused GravNet aggregation and
 the float32 select_with_default kernel.
 """
+import ctypes
 import struct
 import threading
 import weakref
@@ -182,34 +183,42 @@ def _pinned_status(dev: torch.device) -> torch.Tensor:
 
 
 def knn_grad_sorted(grad_distsq: torch.Tensor, nbr_sorted: torch.Tensor, coords: torch.Tensor,
-                    order: torch.Tensor) -> torch.Tensor:
+                    order: torch.Tensor, n_coords: Optional[int] = None,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """d(loss)/d(coords) from d(loss)/d(distsq) with the neighbour rows and permutation of the forward's sorted
-    order (what binned_select_knn keeps for its backward)."""
+    order (what binned_select_knn keeps for its backward).  With `n_coords` the coordinates are the first n_coords
+    columns of the (wider) matrix `coords`, and `out` (same row length as it likes) receives the gradient in its
+    first n_coords columns."""
     _lib.require_device(grad_distsq, nbr_sorted, coords, order)
     L = _lib.lib()
     g = grad_distsq.to(torch.float32).contiguous()
     x = coords.to(torch.float32).contiguous()
-    n, D = x.shape
+    n, ld = x.shape
+    D = ld if n_coords is None else int(n_coords)
     K = nbr_sorted.shape[1]
-    out = torch.empty((n, D), dtype=torch.float32, device=x.device)
+    if out is None:
+        out = torch.empty((n, D), dtype=torch.float32, device=x.device)
     status = torch.zeros(4, dtype=torch.int32, device=x.device)
     ws_bytes = L.fgc_binned_select_knn_grad_sorted_workspace_bytes(n, D)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
-        _lib.check(L.fgc_binned_select_knn_grad_sorted_f32(_lib.ptr(g), _lib.ptr(nbr_sorted), _lib.ptr(x),
-                                                           _lib.ptr(order), _lib.ptr(out), n, K, D, _lib.ptr(status),
-                                                           _lib.ptr(ws), ws_bytes, _lib.stream_ptr()))
+        _lib.check(L.fgc_binned_select_knn_grad_sorted_ld_f32(
+            _lib.ptr(g), _lib.ptr(nbr_sorted), _lib.ptr(x), ld, _lib.ptr(order), _lib.ptr(out), out.stride(0), n, K, D,
+            _lib.ptr(status), _lib.ptr(ws), ws_bytes, _lib.stream_ptr()))
     return out
 
 
-_RS_HOST = {}       # id(tensor) -> (weak reference, version, data pointer, host copy)
+_RS_HOST = {}       # id(tensor) -> (weak reference, version, data pointer, host copy); guarded by _RS_LOCK
+_RS_LOCK = threading.Lock()
+_STATS_LOCK = threading.Lock()
 
 
 def host_row_splits(row_splits: torch.Tensor) -> torch.Tensor:
     """row_splits as an int64 host tensor.  The search is planned on the host, so a device tensor has to be copied
     back, which makes the host wait for everything queued before it.  A model calls the kNN of every layer with the
     same row_splits tensor: the copy is kept for as long as that very tensor object is alive and unmodified
-    (object identity, version counter and data pointer are all checked), so only the first call waits."""
+    (object identity, version counter and data pointer are all checked), so only the first call waits.  The table
+    is shared between host threads under a lock; when it is full the oldest entry goes."""
     if not row_splits.is_cuda:
         return row_splits.detach().to(torch.int64).contiguous()
     try:
@@ -217,14 +226,110 @@ def host_row_splits(row_splits: torch.Tensor) -> torch.Tensor:
     except RuntimeError:          # inference tensors have no version counter: no caching
         return row_splits.detach().to("cpu", torch.int64).contiguous()
     key = id(row_splits)
-    ent = _RS_HOST.get(key)
+    with _RS_LOCK:
+        ent = _RS_HOST.get(key)
     if ent is not None and ent[0]() is row_splits and ent[1] == version and ent[2] == row_splits.data_ptr():
         return ent[3]
-    host = row_splits.detach().to("cpu", torch.int64).contiguous()
-    if len(_RS_HOST) >= 64:
-        _RS_HOST.clear()
-    _RS_HOST[key] = (weakref.ref(row_splits), version, row_splits.data_ptr(), host)
+    host = row_splits.detach().to("cpu", torch.int64).contiguous()     # the wait happens outside the lock
+    with _RS_LOCK:
+        _RS_HOST.pop(key, None)
+        while len(_RS_HOST) >= 64:
+            _RS_HOST.pop(next(iter(_RS_HOST)))                         # dicts keep insertion order: the oldest
+        _RS_HOST[key] = (weakref.ref(row_splits), version, row_splits.data_ptr(), host)
     return host
+
+
+def _knn_forward(coords: torch.Tensor, D: int, row_splits, K: int, direction, n_bins, max_bin_dims: int,
+                 tf_compat: bool, want_backward: bool):
+    """The whole forward of binned_select_knn on the first D columns of the float32 row-major matrix `coords`.
+    Returns (idx, distsq, nbr_sorted, order); the last two (neighbour rows and permutation of the search's sorted
+    order) only when a backward will follow."""
+    L = _lib.lib()
+    dev = coords.device
+    n, ld = coords.shape
+    nbd = min(int(max_bin_dims), D)
+    if nbd < 2 or nbd > 5:
+        raise ValueError("Unsupported number of binning dimensions.")
+    if K < 1 or K > 256:
+        raise ValueError("binned_select_knn on MI355X supports 1 <= K <= 256, got %d" % K)
+    rs_host = host_row_splits(row_splits)
+    n_rs = rs_host.numel()
+    if n_rs < 2:
+        raise ValueError("row_splits needs at least two entries")
+    if n_bins is None or n_bins.numel() == 0:
+        if config.auto_grid:
+            nbd, nb1 = choose_search_grid(rs_host, D, nbd)
+            nb = [nb1] * nbd
+        else:
+            nb = [calculate_optimal_bins(rs_host, K, nbd)] * nbd
+    else:
+        nbt = n_bins.detach().to("cpu", torch.int64)
+        nb = [int(nbt.item())] * nbd if nbt.numel() == 1 else [int(v) for v in nbt.tolist()]
+        if len(nb) != nbd:
+            raise ValueError("bin_by_coordinates: coordinates.size(1) must be equal to nbins.size(0)")
+        if not all(v > 0 for v in nb):
+            raise RuntimeError("BinByCoordinates: n_bins must be greater than zero.")
+    rs_list = rs_host.tolist()
+    if n > 0 and (rs_list[0] != 0 or max(rs_list) != n or rs_list[-1] != n
+                  or any(b < a for a, b in zip(rs_list, rs_list[1:]))):
+        raise RuntimeError("Bin boundaries do not match row splits.")
+    rs_dev = row_splits if (row_splits.is_cuda and row_splits.dtype == torch.int64) else rs_host.to(dev)
+    rs_dev = rs_dev.contiguous()
+    idx = torch.empty((n, K), dtype=torch.int64, device=dev)
+    dist = torch.empty((n, K), dtype=torch.float32, device=dev)
+    order = torch.empty(0, dtype=torch.int32, device=dev)
+    nbr_sorted = None
+    if n > 0:
+        nb_arr = _lib.host_i64(nb)
+        rs_arr = _lib.host_i64(rs_list)
+        ws_bytes = L.fgc_binned_select_knn_workspace_bytes(n, D, nbd, nb_arr, n_rs, K)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        status = torch.zeros(4, dtype=torch.int32, device=dev)
+        stats = torch.zeros(8, dtype=torch.int64, device=dev) if config.collect_stats else None
+        dirt = None
+        if direction is not None and direction.numel() > 0:
+            dirt = direction.to(device=dev, dtype=torch.int64).contiguous()
+        with torch.cuda.device(dev):
+            st = _lib.stream_ptr()
+            # prepare and search are enqueued separately so that the input checks (status word, written by
+            # the prepare stage) can be read back while the search is already queued behind them: the host
+            # then waits for the short prepare stage only and the device never runs dry
+            _lib.check(L.fgc_binned_knn_prepare_ld_f32(
+                _lib.ptr(coords), n, D, ld, _lib.ptr(rs_dev), rs_arr, n_rs, K, nbd, nb_arr, _lib.ptr(dirt),
+                _lib.ptr(status), _lib.ptr(ws), ws_bytes, st))
+            checked = None
+            if config.sync_checks:
+                status_host = _pinned_status(dev)
+                status_host.copy_(status, non_blocking=True)
+                checked = torch.cuda.Event()
+                checked.record()
+            if want_backward:
+                # the backward works in the search's sorted order: it gets the neighbour rows in that order
+                # (int32) and the permutation
+                nbr_sorted = torch.empty((n, K), dtype=torch.int32, device=dev)
+            _lib.check(L.fgc_binned_knn_search_f32(
+                n, D, rs_arr, n_rs, K, nbd, nb_arr, 1 if dirt is not None else 0, 1 if tf_compat else 0,
+                _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(nbr_sorted), _lib.ptr(stats), _lib.ptr(ws), ws_bytes, st))
+            if want_backward:
+                order = torch.empty(n, dtype=torch.int32, device=dev)
+                _lib.check(L.fgc_binned_knn_export_order_i32(n, D, rs_arr, n_rs, K, nbd, nb_arr,
+                                                             1 if dirt is not None else 0, _lib.ptr(ws),
+                                                             ws_bytes, _lib.ptr(order), st))
+        if checked is not None:
+            checked.synchronize()
+            flags = int(status_host[0])
+            if flags & _lib.ST_NONFINITE:
+                raise RuntimeError("BinByCoordinates: input coordinates contain non-finite values")
+            if flags & _lib.ST_BAD_RANGE:
+                raise RuntimeError("BinByCoordinates: dmax_coords must be greater than zero.")
+        if stats is not None:
+            s = stats.tolist()
+            with _STATS_LOCK:
+                last_stats.update(distance_evaluations=s[0], candidate_chunks=s[1], pool_prunes=s[2],
+                                  n_bins=nb, n_vert=n, K=K, n_coords=D)
+    if nbr_sorted is None:
+        nbr_sorted = torch.empty((0, K), dtype=torch.int32, device=dev)
+    return idx, dist, nbr_sorted, order
 
 
 class _BinnedKNN(torch.autograd.Function):
@@ -235,91 +340,9 @@ class _BinnedKNN(torch.autograd.Function):
             raise ValueError("Input coordinates must have at least one dimension.")
         if max_bin_dims <= 0:
             raise ValueError("max_bin_dims must be greater than 0.")
-        L = _lib.lib()
-        dev = coords.device
         coords = coords.to(torch.float32).contiguous()
-        n, D = coords.shape
-        nbd = min(int(max_bin_dims), D)
-        if nbd < 2 or nbd > 5:
-            raise ValueError("Unsupported number of binning dimensions.")
-        if K < 1 or K > 256:
-            raise ValueError("binned_select_knn on MI355X supports 1 <= K <= 256, got %d" % K)
-        rs_host = host_row_splits(row_splits)
-        n_rs = rs_host.numel()
-        if n_rs < 2:
-            raise ValueError("row_splits needs at least two entries")
-        if n_bins is None or n_bins.numel() == 0:
-            if config.auto_grid:
-                nbd, nb1 = choose_search_grid(rs_host, D, nbd)
-                nb = [nb1] * nbd
-            else:
-                nb = [calculate_optimal_bins(rs_host, K, nbd)] * nbd
-        else:
-            nbt = n_bins.detach().to("cpu", torch.int64)
-            nb = [int(nbt.item())] * nbd if nbt.numel() == 1 else [int(v) for v in nbt.tolist()]
-            if len(nb) != nbd:
-                raise ValueError("bin_by_coordinates: coordinates.size(1) must be equal to nbins.size(0)")
-            if not all(v > 0 for v in nb):
-                raise RuntimeError("BinByCoordinates: n_bins must be greater than zero.")
-        rs_list = rs_host.tolist()
-        if n > 0 and (rs_list[0] != 0 or max(rs_list) != n or rs_list[-1] != n
-                      or any(b < a for a, b in zip(rs_list, rs_list[1:]))):
-            raise RuntimeError("Bin boundaries do not match row splits.")
-        rs_dev = row_splits if (row_splits.is_cuda and row_splits.dtype == torch.int64) else rs_host.to(dev)
-        rs_dev = rs_dev.contiguous()
-        idx = torch.empty((n, K), dtype=torch.int64, device=dev)
-        dist = torch.empty((n, K), dtype=torch.float32, device=dev)
-        order = torch.empty(0, dtype=torch.int32, device=dev)
-        nbr_sorted = None
-        if n > 0:
-            nb_arr = _lib.host_i64(nb)
-            rs_arr = _lib.host_i64(rs_list)
-            ws_bytes = L.fgc_binned_select_knn_workspace_bytes(n, D, nbd, nb_arr, n_rs, K)
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-            status = torch.zeros(4, dtype=torch.int32, device=dev)
-            stats = torch.zeros(8, dtype=torch.int64, device=dev) if config.collect_stats else None
-            dirt = None
-            if direction is not None and direction.numel() > 0:
-                dirt = direction.to(device=dev, dtype=torch.int64).contiguous()
-            with torch.cuda.device(dev):
-                st = _lib.stream_ptr()
-                # prepare and search are enqueued separately so that the input checks (status word, written by
-                # the prepare stage) can be read back while the search is already queued behind them: the host
-                # then waits for the short prepare stage only and the device never runs dry
-                _lib.check(L.fgc_binned_knn_prepare_f32(
-                    _lib.ptr(coords), n, D, _lib.ptr(rs_dev), rs_arr, n_rs, K, nbd, nb_arr, _lib.ptr(dirt),
-                    _lib.ptr(status), _lib.ptr(ws), ws_bytes, st))
-                checked = None
-                if config.sync_checks:
-                    status_host = _pinned_status(dev)
-                    status_host.copy_(status, non_blocking=True)
-                    checked = torch.cuda.Event()
-                    checked.record()
-                if ctx.needs_input_grad[0]:
-                    # the backward works in the search's sorted order: it gets the neighbour rows in that order
-                    # (int32) and the permutation
-                    nbr_sorted = torch.empty((n, K), dtype=torch.int32, device=dev)
-                _lib.check(L.fgc_binned_knn_search_f32(
-                    n, D, rs_arr, n_rs, K, nbd, nb_arr, 1 if dirt is not None else 0, 1 if tf_compat else 0,
-                    _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(nbr_sorted), _lib.ptr(stats), _lib.ptr(ws), ws_bytes, st))
-                if ctx.needs_input_grad[0]:
-                    order = torch.empty(n, dtype=torch.int32, device=dev)
-                    _lib.check(L.fgc_binned_knn_export_order_i32(n, D, rs_arr, n_rs, K, nbd, nb_arr,
-                                                                 1 if dirt is not None else 0, _lib.ptr(ws),
-                                                                 ws_bytes, _lib.ptr(order), st))
-            if checked is not None:
-                checked.synchronize()
-                flags = int(status_host[0])
-                if flags & _lib.ST_NONFINITE:
-                    raise RuntimeError("BinByCoordinates: input coordinates contain non-finite values")
-                if flags & _lib.ST_BAD_RANGE:
-                    raise RuntimeError("BinByCoordinates: dmax_coords must be greater than zero.")
-            if stats is not None:
-                s = stats.tolist()
-                last_stats.update(distance_evaluations=s[0], candidate_chunks=s[1], pool_prunes=s[2],
-                                  n_bins=nb, n_vert=n, K=K, n_coords=D)
-        if nbr_sorted is None:
-            nbr_sorted = torch.empty((0, K), dtype=torch.int32, device=dev)
+        idx, dist, nbr_sorted, order = _knn_forward(coords, coords.shape[1], row_splits, K, direction, n_bins,
+                                                    max_bin_dims, tf_compat, ctx.needs_input_grad[0])
         ctx.save_for_backward(nbr_sorted, coords, order)
         ctx.mark_non_differentiable(idx)
         ctx.set_materialize_grads(False)   # no zero tensors for unused output gradients
@@ -464,6 +487,112 @@ class _GravNetAggregate(torch.autograd.Function):
 
 def _gravnet_aggregate_impl(idx, distsq, feat):
     return _GravNetAggregate.apply(idx, distsq, feat)
+
+
+class _GravNetLayerCore(torch.autograd.Function):
+    """kNN in the learned coordinates plus the neighbour aggregation of one GravNet layer (gnn_ops.py:87-102 of the
+    reference) as one autograd node: the aggregation writes (mean | max) side by side into one [N, 2P] matrix for
+    the output layer (no concatenation), and the backward chains the aggregation's gradient with respect to the
+    squared distances straight into the kNN gradient kernel, reading the output layer's input gradient in place
+    (leading dimensions)."""
+
+    @staticmethod
+    def forward(ctx, space, features, row_splits, K):
+        _lib.require_device(space, features)
+        if space.dim() != 2 or features.dim() != 2 or space.shape[0] != features.shape[0] or space.shape[1] == 0:
+            raise ValueError("space must be [N, S] and features [N, P]")
+        L = _lib.lib()
+        coords = space.to(torch.float32).contiguous()
+        feat = features.to(torch.float32).contiguous()
+        n, P = feat.shape
+        dev = feat.device
+        idx, dist, nbr_sorted, order = _knn_forward(coords, coords.shape[1], row_splits, K, None, None, 3, False,
+                                                    ctx.needs_input_grad[0])
+        agg = torch.empty((n, 2 * P), dtype=torch.float32, device=dev)
+        argmax = torch.empty((n, P), dtype=torch.int32, device=dev)
+        if n > 0:
+            with torch.cuda.device(dev):
+                _lib.check(L.fgc_gravnet_aggregate_fwd_ld_f32(
+                    _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(feat), P, n, _lib.ptr(agg),
+                    ctypes.c_void_p(agg.data_ptr() + 4 * P), 2 * P, _lib.ptr(argmax), n, K, P, None,
+                    _lib.stream_ptr()))
+        ctx.save_for_backward(idx, dist, coords, feat, argmax, nbr_sorted, order)
+        ctx.mark_non_differentiable(idx)
+        ctx.set_materialize_grads(False)
+        return idx, dist, agg
+
+    @staticmethod
+    def backward(ctx, _g_idx, g_dist, g_agg):
+        idx, dist, coords, feat, argmax, nbr_sorted, order = ctx.saved_tensors
+        L = _lib.lib()
+        n, P = feat.shape
+        K = idx.shape[1]
+        g_feat = g_dsq = g_space = None
+        if n > 0 and g_agg is not None:
+            if g_agg.dtype != torch.float32 or g_agg.stride(1) != 1:
+                g_agg = g_agg.to(torch.float32).contiguous()
+            g_feat = torch.zeros_like(feat)
+            g_dsq = torch.empty_like(dist)
+            with torch.cuda.device(feat.device):
+                _lib.check(L.fgc_gravnet_aggregate_bwd_ld_f32(
+                    _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(feat), P, n, _lib.ptr(argmax), _lib.ptr(g_agg),
+                    ctypes.c_void_p(g_agg.data_ptr() + 4 * P), g_agg.stride(0), _lib.ptr(g_feat), P, _lib.ptr(g_dsq),
+                    n, K, P, None, _lib.stream_ptr()))
+        if g_dist is not None:
+            g_dsq = g_dist.to(torch.float32) if g_dsq is None else g_dsq + g_dist
+        if ctx.needs_input_grad[0]:
+            g_space = torch.zeros_like(coords) if (g_dsq is None or n == 0) \
+                else knn_grad_sorted(g_dsq, nbr_sorted, coords, order)
+        if not ctx.needs_input_grad[1]:
+            g_feat = None
+        elif g_feat is None:
+            g_feat = torch.zeros_like(feat)
+        return g_space, g_feat, None, None
+
+
+def _gravnet_layer_core_impl(space, features, row_splits, K: int):
+    return _GravNetLayerCore.apply(space, features, row_splits, K)
+
+
+class _DenseSplit(torch.autograd.Function):
+    """y = [x | a] W^T + b without building [x | a]: two products into one output, and in the backward one product
+    for both input gradients (returned as column views of it) and the library's weight-gradient kernel per part."""
+
+    @staticmethod
+    def forward(ctx, x, a, weight, bias):
+        _lib.require_device(x, a, weight)
+        C = x.shape[1]
+        ctx.save_for_backward(x, a, weight)
+        ctx.has_bias = bias is not None
+        w1, w2 = weight[:, :C], weight[:, C:]
+        out = torch.addmm(bias, x, w1.t()) if bias is not None else x.matmul(w1.t())
+        return out.addmm_(a, w2.t())
+
+    @staticmethod
+    def backward(ctx, g):
+        x, a, weight = ctx.saved_tensors
+        if g is None:
+            return None, None, None, None
+        g = g.contiguous()
+        C = x.shape[1]
+        gx = ga = gw = gb = None
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            both = g.matmul(weight)                   # [n, C + A]
+            gx = both[:, :C] if ctx.needs_input_grad[0] else None
+            ga = both[:, C:] if ctx.needs_input_grad[1] else None
+        if ctx.needs_input_grad[2] or (ctx.has_bias and ctx.needs_input_grad[3]):
+            if x.dtype == torch.float32 and a.dtype == torch.float32 and g.dtype == torch.float32:
+                gw1, gb = linear_wgrad(g, x, ctx.has_bias)
+                gw2, _ = linear_wgrad(g, a, False)
+            else:
+                gw1, gw2 = g.t().matmul(x), g.t().matmul(a)
+                gb = g.sum(0) if ctx.has_bias else None
+            gw = torch.cat([gw1, gw2], dim=1)
+        return gx, ga, gw, gb
+
+
+def _dense_split_impl(x, a, weight, bias):
+    return _DenseSplit.apply(x, a, weight, bias)
 
 
 # ------------------------------------------------------------------ object-condensation helper matrices
@@ -705,6 +834,11 @@ def _register():
     lib.impl("gravnet_aggregate", _gravnet_aggregate_impl, "Autograd")
     lib.define("dense(Tensor x, Tensor weight, Tensor? bias) -> Tensor")
     lib.impl("dense", _dense_impl, "Autograd")
+    lib.define("dense_split(Tensor x, Tensor a, Tensor weight, Tensor? bias) -> Tensor")
+    lib.impl("dense_split", _dense_split_impl, "Autograd")
+    lib.define("gravnet_layer_core(Tensor space, Tensor features, Tensor row_splits, int K) -> "
+               "(Tensor, Tensor, Tensor)")
+    lib.impl("gravnet_layer_core", _gravnet_layer_core_impl, "Autograd")
     lib.define("select_with_default_f32(Tensor idx, Tensor feat, float default_value) -> Tensor")
     lib.impl("select_with_default_f32", _select_with_default_impl, "Autograd")
     lib.define("select_with_default_b64(Tensor idx, Tensor feat, float default_value) -> Tensor")

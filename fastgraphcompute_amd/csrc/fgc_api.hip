@@ -138,6 +138,18 @@ extern "C" int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert,
                                           const int64_t *d_direction, int32_t *d_status, void *d_ws,
                                           size_t ws_bytes, void *stream)
 {
+    return fgc_binned_knn_prepare_ld_f32(d_coords, n_vert, n_coords, n_coords, d_row_splits, row_splits_host, n_rs, K,
+                                         n_bin_dims, n_bins, d_direction, d_status, d_ws, ws_bytes, stream);
+}
+
+extern "C" int fgc_binned_knn_prepare_ld_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
+                                             int32_t ld_coords, const int64_t *d_row_splits,
+                                             const int64_t *row_splits_host, int32_t n_rs, int32_t K,
+                                             int32_t n_bin_dims, const int64_t *n_bins,
+                                             const int64_t *d_direction, int32_t *d_status, void *d_ws,
+                                             size_t ws_bytes, void *stream)
+{
+    if (ld_coords < n_coords) return FGC_EINVAL;
     KnnCall c;
     int rc = knn_validate(n_vert, n_coords, row_splits_host, n_rs, K, n_bin_dims, n_bins, d_direction != nullptr,
                           d_ws, ws_bytes, &c);
@@ -153,10 +165,10 @@ extern "C" int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert,
     float *sc = (float *)(ws + w.sc);
     unsigned char *sdir = d_direction ? (unsigned char *)(ws + w.sdir) : nullptr;
 
-    rc = fgc_bin_geometry_f32(d_coords, n_vert, n_coords, n_bin_dims, 2, n_bins, 1, 0.f, 0, geom, d_status,
+    rc = fgc_bin_geometry_f32(d_coords, n_vert, ld_coords, n_bin_dims, 2, n_bins, 1, 0.f, 0, geom, d_status,
                               ws + w.partial, fgc_bin_geometry_workspace_bytes(n_vert), stream);
     if (rc) return rc;
-    rc = fgc_launch_bin_keys(d_coords, (int)n_vert, n_coords, n_bin_dims, c.sub_bits, geom, d_row_splits, n_rs,
+    rc = fgc_launch_bin_keys(d_coords, (int)n_vert, ld_coords, n_bin_dims, c.sub_bits, geom, d_row_splits, n_rs,
                              keys, d_status, s);
     if (rc) return rc;
     uint32_t *skeys = nullptr, *order = nullptr;
@@ -167,7 +179,7 @@ extern "C" int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert,
     if (skeys2 != skeys || order2 != order) return FGC_EINVAL;  // internal layout mismatch
     rc = fgc_launch_bin_boundaries(skeys, (int)n_vert, c.sub_bits * n_bin_dims, (int)c.B, bb, s);
     if (rc) return rc;
-    rc = fgc_launch_gather_sorted(d_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir, s);
+    rc = fgc_launch_gather_sorted(d_coords, ld_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir, s);
     if (rc) return rc;
     return fgc_launch_chunk_boxes(sc, (int)n_vert, n_coords, w.ldc, (float *)(ws + w.box_lo),
                                   (float *)(ws + w.box_hi), (float *)(ws + w.sbox_lo), (float *)(ws + w.sbox_hi), s);

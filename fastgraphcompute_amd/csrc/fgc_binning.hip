@@ -589,7 +589,7 @@ __global__ __launch_bounds__(256) void k_bin_boundaries(const uint32_t *__restri
 }
 
 // sorted structure-of-arrays coordinates: sc[d * ldc + i] = coords[order[i]][d]
-__global__ __launch_bounds__(256) void k_gather_sorted(const float *__restrict__ coords,
+__global__ __launch_bounds__(256) void k_gather_sorted(const float *__restrict__ coords, int ld_in,
                                                        const uint32_t *__restrict__ order, int n, int D,
                                                        int ldc, float *__restrict__ sc,
                                                        const int64_t *__restrict__ direction,
@@ -598,7 +598,7 @@ __global__ __launch_bounds__(256) void k_gather_sorted(const float *__restrict__
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     uint32_t o = order[i];
-    for (int d = 0; d < D; d++) sc[(int64_t)d * ldc + i] = coords[(int64_t)o * D + d];
+    for (int d = 0; d < D; d++) sc[(int64_t)d * ldc + i] = coords[(int64_t)o * ld_in + d];
     if (sdir) {
         int64_t v = direction[o];
         sdir[i] = (unsigned char)((v >= 0 && v <= 2) ? v : 3);
@@ -622,11 +622,11 @@ int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int shift, int n_bin
     return FGC_OK;
 }
 
-int fgc_launch_gather_sorted(const float *coords, const uint32_t *order, int n, int D, int ldc, float *sc,
+int fgc_launch_gather_sorted(const float *coords, int ld_in, const uint32_t *order, int n, int D, int ldc, float *sc,
                              const int64_t *direction, unsigned char *sdir, hipStream_t s)
 {
-    hipLaunchKernelGGL(k_gather_sorted, dim3((unsigned)fgc_cdiv(n, 256)), dim3(256), 0, s, coords, order, n,
-                       D, ldc, sc, direction, sdir);
+    hipLaunchKernelGGL(k_gather_sorted, dim3((unsigned)fgc_cdiv(n, 256)), dim3(256), 0, s, coords, ld_in, order,
+                       n, D, ldc, sc, direction, sdir);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }

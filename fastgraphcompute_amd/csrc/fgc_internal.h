@@ -10,7 +10,7 @@ int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, int sub_b
 int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int shift, int n_bins_total, int *bb, hipStream_t s);
 int fgc_launch_chunk_boxes(const float *sc, int n, int D, int ldc, float *box_lo, float *box_hi, float *sbox_lo,
                            float *sbox_hi, hipStream_t s);
-int fgc_launch_gather_sorted(const float *coords, const uint32_t *order, int n, int D, int ldc, float *sc,
+int fgc_launch_gather_sorted(const float *coords, int ld_in, const uint32_t *order, int n, int D, int ldc, float *sc,
                              const int64_t *direction, unsigned char *sdir, hipStream_t s);
 
 // kNN search over bin-sorted points (fgc_knn.hip)

@@ -270,9 +270,9 @@ extern "C" int fgc_binned_select_knn_grad_f32(const float *d_grad_distsq, const 
 // search wrote in that order (int32, streaming), a padded array-of-points copy of the coordinates in the same
 // order (one 16-byte gather per neighbour and four coordinates), and only the upstream gradient row and the
 // final atomics go through the permutation.
-__global__ __launch_bounds__(256) void k_sorted_points(const float *__restrict__ x, const uint32_t *__restrict__ order,
-                                                       int64_t n, int D, int D4, float4 *__restrict__ xs,
-                                                       float4 *__restrict__ gxs)
+__global__ __launch_bounds__(256) void k_sorted_points(const float *__restrict__ x, int ldx,
+                                                       const uint32_t *__restrict__ order, int64_t n, int D, int D4,
+                                                       float4 *__restrict__ xs, float4 *__restrict__ gxs)
 {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n * D4) return;
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(256) void k_sorted_points(const float *__restrict__
     const int64_t o = order[r];
     float v[4];
 #pragma unroll
-    for (int e = 0; e < 4; e++) v[e] = (c4 * 4 + e < D) ? x[o * D + c4 * 4 + e] : 0.f;
+    for (int e = 0; e < 4; e++) v[e] = (c4 * 4 + e < D) ? x[o * ldx + c4 * 4 + e] : 0.f;
     xs[t] = make_float4(v[0], v[1], v[2], v[3]);
     gxs[t] = make_float4(0.f, 0.f, 0.f, 0.f);       // the gradient accumulator in the same order starts at zero
 }
@@ -530,7 +530,7 @@ __global__ __launch_bounds__(64) void k_knn_grad_sorted(const float *__restrict_
 
 // rows of the sorted-space gradient to the original order: gx[order[r], :] = gxs[r, :D]; one thread per float4 group
 __global__ __launch_bounds__(256) void k_unsort_grad(const float4 *__restrict__ gxs, const uint32_t *__restrict__ order,
-                                                     int64_t n, int D, int D4, float *__restrict__ gx)
+                                                     int64_t n, int D, int D4, float *__restrict__ gx, int ldg)
 {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n * D4) return;
@@ -538,7 +538,7 @@ __global__ __launch_bounds__(256) void k_unsort_grad(const float4 *__restrict__ 
     int c4 = 0;
     if (D4 > 1) { r = t / D4; c4 = (int)(t - r * D4); }
     const float4 v = gxs[t];
-    float *dst = gx + (int64_t)order[r] * D + c4 * 4;
+    float *dst = gx + (int64_t)order[r] * ldg + c4 * 4;
     dst[0] = v.x;
     if (c4 * 4 + 1 < D) dst[1] = v.y;
     if (c4 * 4 + 2 < D) dst[2] = v.z;
@@ -558,6 +558,19 @@ extern "C" int fgc_binned_select_knn_grad_sorted_f32(const float *d_grad_distsq,
                                                      int32_t n_coords, int32_t *d_status, void *d_ws,
                                                      size_t ws_bytes, void *stream)
 {
+    return fgc_binned_select_knn_grad_sorted_ld_f32(d_grad_distsq, d_nbr_sorted, d_coords, n_coords, d_order,
+                                                    d_grad_coords, n_coords, n_vert, K, n_coords, d_status, d_ws,
+                                                    ws_bytes, stream);
+}
+
+extern "C" int fgc_binned_select_knn_grad_sorted_ld_f32(const float *d_grad_distsq, const int32_t *d_nbr_sorted,
+                                                        const float *d_coords, int32_t ld_coords,
+                                                        const int32_t *d_order, float *d_grad_coords,
+                                                        int32_t ld_grad_coords, int64_t n_vert, int32_t K,
+                                                        int32_t n_coords, int32_t *d_status, void *d_ws,
+                                                        size_t ws_bytes, void *stream)
+{
+    if (ld_coords < n_coords || ld_grad_coords < n_coords) return FGC_EINVAL;
     if (n_vert < 0 || K < 1 || n_coords < 1 || n_coords > 128) return FGC_EINVAL;
     if (n_vert >= (1ll << 31) - 1) return FGC_EINVAL;
     if (n_vert == 0) return FGC_OK;
@@ -569,7 +582,7 @@ extern "C" int fgc_binned_select_knn_grad_sorted_f32(const float *d_grad_distsq,
     float4 *xs = (float4 *)d_ws;
     float *gxs = (float *)((char *)d_ws + half);
     hipLaunchKernelGGL(k_sorted_points, dim3((unsigned)fgc_cdiv(n_vert * D4, 256)), dim3(256), 0, s, d_coords,
-                       (const uint32_t *)d_order, n_vert, (int)n_coords, D4, xs, (float4 *)gxs);
+                       (int)ld_coords, (const uint32_t *)d_order, n_vert, (int)n_coords, D4, xs, (float4 *)gxs);
     FGC_LAUNCH_CHECK();
     if (n_coords <= 3) {
         const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GSW);
@@ -585,7 +598,7 @@ extern "C" int fgc_binned_select_knn_grad_sorted_f32(const float *d_grad_distsq,
     }
     FGC_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_unsort_grad, dim3((unsigned)fgc_cdiv(n_vert * D4, 256)), dim3(256), 0, s, (const float4 *)gxs,
-                       (const uint32_t *)d_order, n_vert, (int)n_coords, D4, d_grad_coords);
+                       (const uint32_t *)d_order, n_vert, (int)n_coords, D4, d_grad_coords, (int)ld_grad_coords);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
@@ -675,9 +688,10 @@ extern "C" int fgc_select_with_default_b64(const int64_t *d_idx, const void *d_f
 template <int PW>
 __global__ __launch_bounds__(256) void k_gravnet_fwd(const int64_t *__restrict__ idx,
                                                      const float *__restrict__ dsq,
-                                                     const float *__restrict__ feat, float *__restrict__ fmean,
-                                                     float *__restrict__ fmax, int *__restrict__ argmax,
-                                                     int64_t n, int K, int P)
+                                                     const float *__restrict__ feat, int ldf, int64_t nf,
+                                                     float *__restrict__ fmean, float *__restrict__ fmax, int ldo,
+                                                     int *__restrict__ argmax, int64_t n, int K, int P,
+                                                     int *__restrict__ status)
 {
     constexpr int QPW = 64 / PW;
     const int lane = fgc_lane();
@@ -690,6 +704,7 @@ __global__ __launch_bounds__(256) void k_gravnet_fwd(const int64_t *__restrict__
     // order with the neighbour and its weight broadcast from the lane that fetched them; the gathers of eight
     // slots are in flight together.
     const int gbase = sub * PW;
+    bool bad = false;
     for (int p0 = 0; p0 < P; p0 += PW) {
         const int p = p0 + pl;
         const bool pv = p < P;
@@ -700,7 +715,9 @@ __global__ __launch_bounds__(256) void k_gravnet_fwd(const int64_t *__restrict__
             int m_l = -1;
             float w_l = 0.f;
             if (kk < K) {
-                m_l = (int)idx[i * K + kk];
+                const int64_t mi = idx[i * K + kk];
+                bad = bad || mi >= nf;             // a neighbour past the feature rows: flagged, counts as padding
+                m_l = (mi >= nf) ? -1 : (int)mi;
                 w_l = expf(-10.f * dsq[i * K + kk]);
             }
             const int cnt = min(PW, K - kb);
@@ -711,7 +728,7 @@ __global__ __launch_bounds__(256) void k_gravnet_fwd(const int64_t *__restrict__
                     const int src = gbase + min(j0 + u, PW - 1);
                     const int m = __shfl(m_l, src, 64);
                     w[u] = __shfl(w_l, src, 64);
-                    f[u] = (m >= 0 && pv && j0 + u < cnt) ? feat[(int64_t)m * P + p] : 0.f;
+                    f[u] = (m >= 0 && pv && j0 + u < cnt) ? feat[(int64_t)m * ldf + p] : 0.f;
                 }
 #pragma unroll
                 for (int u = 0; u < 8; u++) {
@@ -724,21 +741,24 @@ __global__ __launch_bounds__(256) void k_gravnet_fwd(const int64_t *__restrict__
             }
         }
         if (pv) {
-            fmean[i * P + p] = s / (float)K;
-            fmax[i * P + p] = mx;
+            fmean[i * ldo + p] = s / (float)K;
+            fmax[i * ldo + p] = mx;
             if (argmax) argmax[i * P + p] = am;
         }
     }
+    if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
 }
 
 template <int PW>
 __global__ __launch_bounds__(256) void k_gravnet_bwd(const int64_t *__restrict__ idx,
                                                      const float *__restrict__ dsq,
-                                                     const float *__restrict__ feat,
+                                                     const float *__restrict__ feat, int ldf, int64_t nf,
                                                      const int *__restrict__ argmax,
                                                      const float *__restrict__ gmean,
-                                                     const float *__restrict__ gmax, float *__restrict__ gfeat,
-                                                     float *__restrict__ gdsq, int64_t n, int K, int P)
+                                                     const float *__restrict__ gmax, int ldg,
+                                                     float *__restrict__ gfeat, int ldgf,
+                                                     float *__restrict__ gdsq, int64_t n, int K, int P,
+                                                     int *__restrict__ status)
 {
     constexpr int QPW = 64 / PW;
     const int lane = fgc_lane();
@@ -753,12 +773,13 @@ __global__ __launch_bounds__(256) void k_gravnet_bwd(const int64_t *__restrict__
     // flight together), adds w * c to their feature gradients and keeps one partial dot product per slot; an
     // exchange across the group's lanes (plain butterflies down to 8 lanes, then halving) leaves the dot
     // product of slot j0 + (lane & 7) in every lane, and the lane that fetched that slot writes grad_distsq.
+    bool bad = false;
     const bool single = P <= PW;      // one feature per lane: its upstream gradients stay in registers
     float cm0 = 0.f, gx0 = 0.f;
     int am0 = -1;
     if (single && qv && pl < P) {
-        cm0 = gmean[i * P + pl] * invK;
-        gx0 = gmax[i * P + pl];
+        cm0 = gmean[i * ldg + pl] * invK;
+        gx0 = gmax[i * ldg + pl];
         am0 = argmax[i * P + pl];
     }
     for (int kb = 0; kb < K; kb += PW) {
@@ -766,7 +787,9 @@ __global__ __launch_bounds__(256) void k_gravnet_bwd(const int64_t *__restrict__
         int m_l = -1;
         float w_l = 0.f;
         if (qv && kk < K) {
-            m_l = (int)idx[i * K + kk];
+            const int64_t mi = idx[i * K + kk];
+            bad = bad || mi >= nf;                 // as in the forward: flagged, counts as padding
+            m_l = (mi >= nf) ? -1 : (int)mi;
             w_l = expf(-10.f * dsq[i * K + kk]);
         }
         const int cnt = min(PW, K - kb);
@@ -787,19 +810,19 @@ __global__ __launch_bounds__(256) void k_gravnet_bwd(const int64_t *__restrict__
                 float cm = cm0, gx = gx0;
                 int am = am0;
                 if (!single) {
-                    cm = pv ? gmean[i * P + p] * invK : 0.f;
-                    gx = pv ? gmax[i * P + p] : 0.f;
+                    cm = pv ? gmean[i * ldg + p] * invK : 0.f;
+                    gx = pv ? gmax[i * ldg + p] : 0.f;
                     am = pv ? argmax[i * P + p] : -1;
                 }
                 float f[8];
 #pragma unroll
-                for (int u = 0; u < 8; u++) f[u] = (m[u] >= 0 && pv) ? feat[(int64_t)m[u] * P + p] : 0.f;
+                for (int u = 0; u < 8; u++) f[u] = (m[u] >= 0 && pv) ? feat[(int64_t)m[u] * ldf + p] : 0.f;
 #pragma unroll
                 for (int u = 0; u < 8; u++) {
                     if (m[u] >= 0 && pv) {
                         const float c = cm + (am == kb + j0 + u ? gx : 0.f);
                         vals[u] += f[u] * c;
-                        atomicAdd(&gfeat[(int64_t)m[u] * P + p], w[u] * c);
+                        atomicAdd(&gfeat[(int64_t)m[u] * ldgf + p], w[u] * c);
                     }
                 }
             }
@@ -821,6 +844,7 @@ __global__ __launch_bounds__(256) void k_gravnet_bwd(const int64_t *__restrict__
             if (qv && (pl & ~7) == j0 && kk < K) gdsq[i * K + kk] = -10.f * w_l * vals[0];
         }
     }
+    if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
 }
 
 static int pick_pw(int P)
@@ -834,14 +858,24 @@ extern "C" int fgc_gravnet_aggregate_fwd_f32(const int64_t *d_idx, const float *
                                              float *d_fmean, float *d_fmax, int32_t *d_argmax, int64_t n_vert,
                                              int32_t K, int32_t P, void *stream)
 {
-    if (n_vert < 0 || K < 1 || P < 1) return FGC_EINVAL;
+    return fgc_gravnet_aggregate_fwd_ld_f32(d_idx, d_distsq, d_feat, P, n_vert, d_fmean, d_fmax, P, d_argmax, n_vert, K,
+                                            P, nullptr, stream);
+}
+
+extern "C" int fgc_gravnet_aggregate_fwd_ld_f32(const int64_t *d_idx, const float *d_distsq, const float *d_feat,
+                                                int32_t ld_feat, int64_t n_feat_rows, float *d_fmean,
+                                                float *d_fmax, int32_t ld_out, int32_t *d_argmax, int64_t n_vert,
+                                                int32_t K, int32_t P, int32_t *d_status, void *stream)
+{
+    if (n_vert < 0 || K < 1 || P < 1 || ld_feat < P || ld_out < P || n_feat_rows < 0) return FGC_EINVAL;
     if (n_vert == 0) return FGC_OK;
     hipStream_t s = (hipStream_t)stream;
     const int pw = pick_pw(P);
     const unsigned blocks = (unsigned)fgc_cdiv(fgc_cdiv(n_vert, 64 / pw), 4);
 #define FGC_L(PWW)                                                                                    \
     hipLaunchKernelGGL((k_gravnet_fwd<PWW>), dim3(blocks), dim3(256), 0, s, d_idx, d_distsq, d_feat, \
-                       d_fmean, d_fmax, d_argmax, n_vert, (int)K, (int)P)
+                       (int)ld_feat, n_feat_rows, d_fmean, d_fmax, (int)ld_out, d_argmax, n_vert, (int)K, (int)P, \
+                       d_status)
     switch (pw) {
     case 8: FGC_L(8); break;
     case 16: FGC_L(16); break;
@@ -858,15 +892,27 @@ extern "C" int fgc_gravnet_aggregate_bwd_f32(const int64_t *d_idx, const float *
                                              const float *d_grad_fmax, float *d_grad_feat, float *d_grad_distsq,
                                              int64_t n_vert, int32_t K, int32_t P, void *stream)
 {
-    if (n_vert < 0 || K < 1 || P < 1) return FGC_EINVAL;
+    return fgc_gravnet_aggregate_bwd_ld_f32(d_idx, d_distsq, d_feat, P, n_vert, d_argmax, d_grad_fmean, d_grad_fmax, P,
+                                            d_grad_feat, P, d_grad_distsq, n_vert, K, P, nullptr, stream);
+}
+
+extern "C" int fgc_gravnet_aggregate_bwd_ld_f32(const int64_t *d_idx, const float *d_distsq, const float *d_feat,
+                                                int32_t ld_feat, int64_t n_feat_rows, const int32_t *d_argmax,
+                                                const float *d_grad_fmean, const float *d_grad_fmax,
+                                                int32_t ld_grad, float *d_grad_feat, int32_t ld_grad_feat,
+                                                float *d_grad_distsq, int64_t n_vert, int32_t K, int32_t P,
+                                                int32_t *d_status, void *stream)
+{
+    if (n_vert < 0 || K < 1 || P < 1 || ld_feat < P || ld_grad < P || ld_grad_feat < P || n_feat_rows < 0)
+        return FGC_EINVAL;
     if (n_vert == 0) return FGC_OK;
     hipStream_t s = (hipStream_t)stream;
     const int pw = pick_pw(P);
     const unsigned blocks = (unsigned)fgc_cdiv(fgc_cdiv(n_vert, 64 / pw), 4);
-#define FGC_L(PWW)                                                                                     \
-    hipLaunchKernelGGL((k_gravnet_bwd<PWW>), dim3(blocks), dim3(256), 0, s, d_idx, d_distsq, d_feat,  \
-                       d_argmax, d_grad_fmean, d_grad_fmax, d_grad_feat, d_grad_distsq, n_vert, (int)K, \
-                       (int)P)
+#define FGC_L(PWW)                                                                                         \
+    hipLaunchKernelGGL((k_gravnet_bwd<PWW>), dim3(blocks), dim3(256), 0, s, d_idx, d_distsq, d_feat,      \
+                       (int)ld_feat, n_feat_rows, d_argmax, d_grad_fmean, d_grad_fmax, (int)ld_grad, d_grad_feat, \
+                       (int)ld_grad_feat, d_grad_distsq, n_vert, (int)K, (int)P, d_status)
     switch (pw) {
     case 8: FGC_L(8); break;
     case 16: FGC_L(16); break;

@@ -26,6 +26,20 @@ def dense(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -
     return torch.ops.fastgraphcompute_custom_ops.dense(x, weight, bias)
 
 
+@torch.jit.script
+def dense_split(x: torch.Tensor, a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """cat([x, a], 1) W^T + b without the concatenation (weight is [out, x.shape[1] + a.shape[1]])."""
+    return torch.ops.fastgraphcompute_custom_ops.dense_split(x, a, weight, bias)
+
+
+@torch.jit.script
+def gravnet_layer_core(space: torch.Tensor, features: torch.Tensor, row_splits: torch.Tensor,
+                       k: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """kNN in `space` and aggregation of `features` over the neighbours as one autograd node:
+    (neighbor_idx [N, k], distsq [N, k], [N, 2P] = mean | max of features * exp(-10 distsq))."""
+    return torch.ops.fastgraphcompute_custom_ops.gravnet_layer_core(space, features, row_splits, k)
+
+
 class Dense(torch.nn.Linear):
     """torch.nn.Linear (same parameters, state_dict and results) whose weight gradient is the library's split
     reduction over the points.  For the layers around GravNetOp in a point-cloud model: their weight-gradient
@@ -68,16 +82,14 @@ class GravNetOp(torch.nn.Module):
         self.optimization_arguments = optimization_arguments
 
     def forward(self, x: torch.Tensor, row_splits: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-        # both projections of x in one product (x is read once, one weight-gradient reduction in the backward)
-        n_space = self.space_transformations.weight.shape[0]
-        w = torch.cat([self.space_transformations.weight, self.propagate_transformations.weight], dim=0)
-        b = torch.cat([self.space_transformations.bias, self.propagate_transformations.bias], dim=0)
-        projected = dense(x, w, b)
-        space = projected[:, :n_space].contiguous()
-        propagate = projected[:, n_space:].contiguous()
-        neighbor_idx, distsq = binned_select_knn(self.k, space, row_splits)
-        fmean, fmax = gravnet_aggregate(neighbor_idx, distsq, propagate)
-        output = torch.cat([x, fmean, fmax], dim=1)
+        # The two projections are separate products, so that the coordinates and the features are matrices of
+        # their own (rows of the features aligned to their 128 bytes: the aggregation gathers and, in the backward,
+        # updates whole rows); search and aggregation are one autograd node that writes (mean | max) side by side,
+        # and the output layer multiplies x and that matrix by its two weight blocks - no slice copies and no
+        # concatenation, forward or backward.
+        space = dense(x, self.space_transformations.weight, self.space_transformations.bias)
+        propagate = dense(x, self.propagate_transformations.weight, self.propagate_transformations.bias)
+        neighbor_idx, distsq, aggregated = gravnet_layer_core(space, propagate, row_splits, self.k)
         lin = self.output_transformations[0]
-        out = self.output_transformations[1](dense(output, lin.weight, lin.bias))
+        out = self.output_transformations[1](dense_split(x, aggregated, lin.weight, lin.bias))
         return out, neighbor_idx, distsq, space

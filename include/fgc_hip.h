@@ -166,6 +166,14 @@ int fgc_binned_knn_prepare_f32(const float *d_coords, int64_t n_vert, int32_t n_
                                int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
                                const int64_t *d_direction, int32_t *d_status, void *d_ws,
                                size_t ws_bytes, void *stream);
+/* fgc_binned_knn_prepare_f32 for coordinates that are the first n_coords columns of a wider row-major matrix
+ * (ld_coords floats per row), e.g. the learned coordinates inside the joint projection of a GravNet layer
+ * (gnn_ops.py:79-87 computes them as a matrix of their own). */
+int fgc_binned_knn_prepare_ld_f32(const float *d_coords, int64_t n_vert, int32_t n_coords, int32_t ld_coords,
+                                  const int64_t *d_row_splits, const int64_t *row_splits_host, int32_t n_rs,
+                                  int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
+                                  const int64_t *d_direction, int32_t *d_status, void *d_ws, size_t ws_bytes,
+                                  void *stream);
 int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
                               int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
                               int32_t with_direction, int32_t tf_compat, int64_t *d_idx,
@@ -233,6 +241,14 @@ int fgc_binned_select_knn_grad_sorted_f32(const float *d_grad_distsq, const int3
                                           int64_t n_vert, int32_t K, int32_t n_coords, int32_t *d_status,
                                           void *d_ws, size_t ws_bytes, void *stream);
 
+/* The same with leading dimensions: d_coords and d_grad_coords are the first n_coords columns of row-major
+ * matrices with ld_coords / ld_grad_coords floats per row (the other columns of d_grad_coords are not touched). */
+int fgc_binned_select_knn_grad_sorted_ld_f32(const float *d_grad_distsq, const int32_t *d_nbr_sorted,
+                                             const float *d_coords, int32_t ld_coords, const int32_t *d_order,
+                                             float *d_grad_coords, int32_t ld_grad_coords, int64_t n_vert,
+                                             int32_t K, int32_t n_coords, int32_t *d_status, void *d_ws,
+                                             size_t ws_bytes, void *stream);
+
 /* ---------------------------------------------------------------------------
  * Replaces select_with_default (oc_helper.py:232-271) for float32 features:
  * out[v,k,:] = feat[idx[v,k],:], or default_value where idx[v,k] == -1.
@@ -267,6 +283,21 @@ int fgc_gravnet_aggregate_bwd_f32(const int64_t *d_idx, const float *d_distsq,
                                   const float *d_grad_fmean, const float *d_grad_fmax,
                                   float *d_grad_feat, float *d_grad_distsq, int64_t n_vert,
                                   int32_t K, int32_t P, void *stream);
+
+/* The same with leading dimensions, so that the layer around the aggregation needs no copies: the features may
+ * be columns of a wider matrix (ld_feat floats per row, n_feat_rows rows; gnn_ops.py:83 computes them as a matrix
+ * of their own), d_fmean / d_fmax may point into one [n_vert, 2P] matrix that feeds the output layer directly
+ * (ld_out; replaces the torch.cat of gnn_ops.py:105), the gradients come from and go to such matrices likewise.
+ * A neighbour index >= n_feat_rows sets FGC_ST_BAD_INDEX in d_status (optional) and counts as padding. */
+int fgc_gravnet_aggregate_fwd_ld_f32(const int64_t *d_idx, const float *d_distsq, const float *d_feat,
+                                     int32_t ld_feat, int64_t n_feat_rows, float *d_fmean, float *d_fmax,
+                                     int32_t ld_out, int32_t *d_argmax, int64_t n_vert, int32_t K, int32_t P,
+                                     int32_t *d_status, void *stream);
+int fgc_gravnet_aggregate_bwd_ld_f32(const int64_t *d_idx, const float *d_distsq, const float *d_feat,
+                                     int32_t ld_feat, int64_t n_feat_rows, const int32_t *d_argmax,
+                                     const float *d_grad_fmean, const float *d_grad_fmax, int32_t ld_grad,
+                                     float *d_grad_feat, int32_t ld_grad_feat, float *d_grad_distsq,
+                                     int64_t n_vert, int32_t K, int32_t P, int32_t *d_status, void *stream);
 
 /* ---------------------------------------------------------------------------
  * Weight and bias gradient of a dense layer y = x W^T + b over n points:
