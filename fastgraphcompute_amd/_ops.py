@@ -250,8 +250,8 @@ def _knn_forward(coords: torch.Tensor, D: int, row_splits, K: int, direction, n_
     nbd = min(int(max_bin_dims), D)
     if nbd < 2 or nbd > 5:
         raise ValueError("Unsupported number of binning dimensions.")
-    if K < 1 or K > 256:
-        raise ValueError("binned_select_knn on MI355X supports 1 <= K <= 256, got %d" % K)
+    if K < 1 or K > 1024:
+        raise ValueError("binned_select_knn on MI355X supports 1 <= K <= 1024, got %d" % K)
     rs_host = host_row_splits(row_splits)
     n_rs = rs_host.numel()
     if n_rs < 2:
@@ -714,8 +714,8 @@ def _select_knn_impl(coords: torch.Tensor, row_splits: torch.Tensor, mask: torch
     if coords.dim() != 2 or coords.shape[1] == 0:
         raise ValueError("coords must be [n_vert, n_coords]")
     K = int(n_neighbours)
-    if K < 1 or K > 256:
-        raise ValueError("select_knn on MI355X supports 1 <= n_neighbours <= 256, got %d" % K)
+    if K < 1 or K > 1024:
+        raise ValueError("select_knn on MI355X supports 1 <= n_neighbours <= 1024, got %d" % K)
     L = _lib.lib()
     dev = coords.device
     x = coords.to(torch.float32).contiguous()

@@ -754,6 +754,14 @@ template <int NSEG> static int launch_knn_r(const KnnArgs &a, hipStream_t s)
     return launch_knn_d<NSEG, 4>(a, s);
 }
 
+template <int NSEG> static int launch_knn_big(const KnnArgs &a, hipStream_t s)
+{
+    if (a.nbd <= 2) return launch_knn_t<0, NSEG, 1>(a, s);
+    if (a.nbd == 3) return launch_knn_t<0, NSEG, 2>(a, s);
+    if (a.nbd == 4) return launch_knn_t<0, NSEG, 3>(a, s);
+    return launch_knn_t<0, NSEG, 4>(a, s);
+}
+
 int fgc_launch_knn(const KnnArgs &a_in, hipStream_t s)
 {
     KnnArgs a = a_in;
@@ -765,5 +773,9 @@ int fgc_launch_knn(const KnnArgs &a_in, hipStream_t s)
     a.pool_cap = ((a.K + (a.K <= 64 ? POOL_EXTRA_SMALL_K : POOL_EXTRA) + 15) / 16) * 16;
     if (a.K <= 64) return launch_knn_r<1>(a, s);
     if (a.K <= 128) return launch_knn_r<2>(a, s);
-    return launch_knn_r<4>(a, s);
+    if (a.K <= 256) return launch_knn_r<4>(a, s);
+    // Beyond 256 neighbours (rare: the reference's benchmarks stop at 100) only the variant that reads the
+    // coordinates from memory per evaluation is built, with pools of up to 1072 entries per query.
+    if (a.K <= 512) return launch_knn_big<8>(a, s);
+    return launch_knn_big<16>(a, s);
 }

@@ -35,7 +35,9 @@ extern "C" {
 #define FGC_ETOOLARGE (-4)   /* input exceeds the fixed scratch of a no-allocation entry point */
 
 #define FGC_MAX_BIN_DIMS 5
-#define FGC_MAX_K 256        /* neighbours per query the kNN kernel supports  */
+#define FGC_MAX_K 1024       /* neighbours per query the kNN kernels support; the reference's loops take any
+                                K (binned_select_knn_cpu.cpp:211-326), its benchmarks stop at 100.  Up to 256
+                                the search runs its register-tiled kernels, beyond that a slower variant  */
 #define FGC_STATUS_WORDS 4
 /* bits of d_status[0] */
 #define FGC_ST_NONFINITE 1   /* a binned coordinate is inf/nan                */

@@ -39,7 +39,7 @@ def test_argument_validation_without_device():
 
     def call(n=100, D=3, K=8, nbd=3, rs_=rs, n_rs=2, ws_bytes=ws, nb_=nb):
         return L.fgc_binned_knn_search_f32(n, D, rs_, n_rs, K, nbd, nb_, 0, 0, fake, fake, None, None, fake, ws_bytes, None)
-    assert call(K=0) == -1 and call(K=257) == -1
+    assert call(K=0) == -1 and call(K=1025) == -1
     assert call(nbd=1) == -3 and call(nbd=6) == -3 and call(D=2, nbd=3) == -3
     assert call(rs_=_lib.host_i64([0, 99])) == -1            # row splits do not end at n_vert
     assert call(rs_=_lib.host_i64([0, 120, 100]), n_rs=3) == -1

@@ -70,6 +70,31 @@ def test_neighbour_counts(oracle, K):
     _check(oracle, K, coords, [0, 1200, 2500])
 
 
+@pytest.mark.parametrize("K,D", [(257, 3), (400, 2), (512, 4), (513, 3), (700, 6), (1024, 3)])
+def test_more_than_256_neighbours(oracle, K, D):
+    # beyond 256 neighbours the search runs its slower any-K variant; one event smaller than K (padding) and the
+    # gradient through the op's backward
+    rng = np.random.default_rng(K + D)
+    n = 2600
+    coords = rng.random((n, D)).astype(np.float32)
+    rs = [0, 1500, 1500 + 300, n]
+    gi, gd = _check(oracle, K, coords, rs)
+    check_knn_properties(gi, gd, coords, rs, K)
+    from fastgraphcompute_amd import binned_select_knn
+    x = torch.from_numpy(coords).cuda().requires_grad_(True)
+    idx, dist = binned_select_knn(K, x, torch.tensor(rs, device="cuda"))
+    up = rng.standard_normal((n, K)).astype(np.float32)
+    dist.backward(torch.from_numpy(up).cuda())
+    exp = oracle.knn_grad(up, idx.cpu().numpy(), coords)
+    assert np.abs(x.grad.cpu().numpy() - exp).max() <= 1e-5 * np.abs(exp).max()
+
+
+def test_neighbour_count_limit():
+    from fastgraphcompute_amd import binned_select_knn
+    with pytest.raises((ValueError, RuntimeError)):
+        binned_select_knn(1025, torch.rand(3000, 3, device="cuda"), torch.tensor([0, 3000], device="cuda"))
+
+
 @pytest.mark.parametrize("mbd", [2, 3, 4, 5])
 def test_max_bin_dims(oracle, mbd):
     rng = np.random.default_rng(80 + mbd)
