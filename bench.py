@@ -21,6 +21,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 N_SIMD = 1024           # 256 compute units x 4 SIMDs; a VALU wavefront instruction occupies its SIMD for 4 cycles
+GPU_CLOCK_HZ = 2.4e9    # MI355X peak engine clock (published); used only to turn instruction counts into a time share
 
 
 def profile_facts():
@@ -82,6 +83,8 @@ def main():
     ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "oc_helper", "gravnet_model"])
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="skip the short GravNetOp / model-step measurements appended to the default line")
     ap.add_argument("--cpu-sample-seconds", type=float, default=15.0)
     ap.add_argument("--cpu-reference-full", action="store_true",
                     help="also time the reference's own compiled CPU kernel (oracle/_ref) on ALL queries of the "
@@ -108,12 +111,15 @@ def main():
     L = _lib.lib()
 
     if args.workload == "oc_helper":
-        return oc_helper_workload(args, dev)
+        print(json.dumps(oc_helper_workload(args, dev)), flush=True)
+        return
     if args.workload == "gravnet_model":
-        return gravnet_model_workload(args, dev)
+        print(json.dumps(gravnet_model_workload(args, dev)), flush=True)
+        return
     w = workloads.CONFIGS[args.workload](args.scale)
     if args.workload == "cfg3":
-        return gravnet_workload(args, w, dev)
+        print(json.dumps(gravnet_workload(args, w, dev)), flush=True)
+        return
     K = int(w["K"])
     coords_h = w["coords"]
     n, D = coords_h.shape
@@ -198,7 +204,7 @@ def main():
     # algorithmic bytes of one search launch: every distance evaluation reads one
     # D-float candidate, every query is read once, every (idx, distsq) slot written once
     facts = profile_facts() if args.scale == 1.0 else {}
-    clock_hz = torch.cuda.get_device_properties(dev).clock_rate * 1e3
+    clock_hz = GPU_CLOCK_HZ
     bytes_alg = 4.0 * D * c_eval + 4.0 * D * n + 12.0 * K * n
     # VALU wavefront instructions that are distance arithmetic: per 64 evaluations D subtractions, D
     # multiplications, D - 1 additions, the compare, and the D + 1 broadcasts of the query and its bound
@@ -243,6 +249,20 @@ def main():
         result["cpu_baseline"], result["cpu_baseline_allcores"] = cpu_baseline(w, K, n, args.cpu_sample_seconds)
     if args.cpu_reference_full:
         result["cpu_baseline_reference_full"] = cpu_reference_full(w, K, n)
+    if args.workload == "cfg4" and args.scale == 1.0 and not args.no_secondary:
+        # the steps either side of the path, a few iterations each: the GravNetOp layer at the cfg3 shape and the
+        # training step of the reference's 4-layer model benchmark
+        del coords, coords_g, grad_d, ws
+        torch.cuda.empty_cache()
+        sub = argparse.Namespace(**vars(args))
+        sub.steps, sub.warmup = 5, 2
+        g = gravnet_workload(sub, workloads.CONFIGS["cfg3"](1.0), dev)
+        m = gravnet_model_workload(sub, dev)
+        result["secondary"] = {
+            "cfg3_gravnet_op_ms_per_step": g["ms_per_step"], "cfg3_stages_ms": g["stages_ms"],
+            "cfg3_roofline_aggregate_bwd": {k: g["roofline"][k] for k in ("achieved", "frac", "kernel_ms")},
+            "gravnet_model_ms_per_step": m["ms_per_step"],
+            "gravnet_model_ms_per_step_with_use_dense_layers": m["ms_per_step_with_use_dense_layers"]}
     print(json.dumps(result), flush=True)
 
 
@@ -272,11 +292,65 @@ def gravnet_workload(args, w, dev):
     torch.cuda.synchronize()
     t = (time.perf_counter() - t0) / args.steps
     n = w["x"].shape[0]
-    print(json.dumps({
+    result = {
         "metric": "GravNetOp forward+backward points/sec", "value": round(n / t, 1), "unit": "points/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(t * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": w["name"], "n_points": n, "events": 2}}), flush=True)
+        "config": {"workload": w["name"], "n_points": n, "events": 2}}
+    result.update(gravnet_stage_times(op, x, rs, w, dev))
+    return result
+
+
+def gravnet_stage_times(op, x, rs, w, dev):
+    """The two aggregation kernels of the layer on their own (events on the launch stream, through the C ABI) and
+    the roofline entry of the backward one, the largest kernel of the step."""
+    import ctypes
+    import numpy as np
+    import torch
+    from fastgraphcompute_amd import _lib
+    L = _lib.lib()
+    with torch.no_grad():
+        space = op.space_transformations(x).contiguous()
+        feat = op.propagate_transformations(x).contiguous()
+    import fastgraphcompute_amd as fgc
+    idx, dist = fgc.binned_select_knn(int(w["K"]), space, rs)
+    n, K = idx.shape
+    P = feat.shape[1]
+    agg = torch.empty((n, 2 * P), device=dev)
+    am = torch.empty((n, P), dtype=torch.int32, device=dev)
+    g_agg = torch.randn((n, 2 * P), device=dev)
+    g_feat = torch.zeros((n, P), device=dev)
+    g_dsq = torch.empty((n, K), device=dev)
+    st = _lib.stream_ptr()
+
+    def fwd():
+        _lib.check(L.fgc_gravnet_aggregate_fwd_ld_f32(_lib.ptr(idx), _lib.ptr(dist), _lib.ptr(feat), P, n, _lib.ptr(agg),
+                                                      ctypes.c_void_p(agg.data_ptr() + 4 * P), 2 * P, _lib.ptr(am), n,
+                                                      K, P, None, st))
+
+    def bwd():
+        _lib.check(L.fgc_gravnet_aggregate_bwd_ld_f32(_lib.ptr(idx), _lib.ptr(dist), _lib.ptr(feat), P, n, _lib.ptr(am),
+                                                      _lib.ptr(g_agg), ctypes.c_void_p(g_agg.data_ptr() + 4 * P),
+                                                      2 * P, _lib.ptr(g_feat), P, _lib.ptr(g_dsq), n, K, P, None, st))
+
+    def timed(fn, reps=8):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for a, b in ev:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        return float(np.median([a.elapsed_time(b) for a, b in ev][2:]))
+
+    t_fwd, t_bwd = timed(fwd), timed(bwd)
+    clock_hz = GPU_CLOCK_HZ
+    facts = profile_facts()
+    # index + distance rows, one P-float gather per pair, features / outputs once; the backward gathers and scatters
+    fwd_alg = 12.0 * K * n + 4.0 * P * n * K + 8.0 * P * n
+    bwd_alg = fwd_alg + 4.0 * P * n * K
+    return {"stages_ms": {"aggregate_fwd": round(t_fwd, 4), "aggregate_bwd": round(t_bwd, 4)},
+            "roofline": roofline_entry("k_gravnet_bwd", w["name"], bwd_alg, t_bwd, clock_hz, None, facts),
+            "roofline_aggregate_fwd": roofline_entry("k_gravnet_fwd", w["name"], fwd_alg, t_fwd, clock_hz, None, facts)}
 
 
 def gravnet_model_workload(args, dev):
@@ -336,12 +410,12 @@ def gravnet_model_workload(args, dev):
     from fastgraphcompute_amd.gnn_ops import use_dense_layers
     use_dense_layers(model)                # same parameters, weight gradients by the library's kernel
     t_dense = timed_steps()
-    print(json.dumps({
+    return {
         "metric": "GravNet model training step nodes/sec", "value": round(n / t, 1), "unit": "nodes/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(t * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "gravnet_model_4layers_h128_k64", "n_points": n, "events": 1},
-        "ms_per_step_with_use_dense_layers": round(t_dense * 1e3, 4)}), flush=True)
+        "ms_per_step_with_use_dense_layers": round(t_dense * 1e3, 4)}
 
 
 def oc_helper_workload(args, dev):
@@ -423,7 +497,7 @@ def oc_helper_workload(args, dev):
         result["cpu_baseline"] = {"value": round(n * (sel.size / uv.size) / tc, 1), "unit": "vertices/s", "cores": 1,
                                   "kind": "port", "sample": "calc_m restatement on %d of %d objects (%.2f s per pass, 3 passes), "
                                   "object analysis excluded" % (sel.size, uv.size, tc)}
-    print(json.dumps(result), flush=True)
+    return result
 
 
 def cpu_reference_full(w, K, n):

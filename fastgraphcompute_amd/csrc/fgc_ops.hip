@@ -485,11 +485,7 @@ __global__ __launch_bounds__(64) void k_knn_grad_sorted(const float *__restrict_
                     vals[sl[u] * D4 + c4] = v;
                 }
                 const bool ovf = m[u] >= 0 && sl[u] < 0;
-#ifndef GRAD_ABL_NOOVF
                 const unsigned long long om = fgc_ballot(ovf);
-#else
-                const unsigned long long om = fgc_ballot(ovf && add.x == 123.456f);
-#endif
                 if (om) {
                     // float4 groups leave in pairs (one 32-byte update per target), an unpaired last one alone
                     if (!PACK && !(c4 & 1) && c4 + 1 < D4) addp[u] = add;
@@ -516,11 +512,7 @@ __global__ __launch_bounds__(64) void k_knn_grad_sorted(const float *__restrict_
         const unsigned m = tags[sl * KS];
         if (m == GRAD_EMPTY || c >= D) continue;
         const float v = vflat[t];
-#ifndef GRAD_ABL_NOFLUSH
         if (v != 0.f) atomicAdd(&gxs[(int64_t)m * ld + c], v);
-#else
-        if (v == 123.456f) atomicAdd(&gxs[(int64_t)m * ld + c], v);
-#endif
     }
     if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
 #ifdef FGC_GRAD_COUNTERS
