@@ -216,7 +216,12 @@ def main():
     # gradient kernel: upstream gradient + neighbour rows + one D-float gather per pair + coordinates in, gradient out
     grad_alg = 4.0 * K * n + 8.0 * K * n + 4.0 * D * n * K + 8.0 * D * n
     roofline_grad = roofline_entry("k_knn_grad_sorted", w["name"], grad_alg, t_grad, clock_hz, None, facts)
-    roofline_grad["kernel_ms_includes"] = "sorted copy of the points, the gradient kernel, un-sort of the result"
+    roofline_grad["kernel_ms_includes"] = "k_sorted_points, k_knn_grad_sorted, k_unsort_grad (one library call)"
+    if roofline_grad["traffic"] is not None:       # the two small kernels of the same call move bytes too
+        extra = sum(facts.get((k, w["name"]), {}).get("traffic_bytes", 0.0) for k in ("k_sorted_points", "k_unsort_grad"))
+        roofline_grad["traffic"] += extra
+        roofline_grad["physical_gbs"] = round(roofline_grad["traffic"] / (t_grad * 1e-3) / 1e9, 1)
+        roofline_grad["physical_frac"] = round(roofline_grad["physical_gbs"] / HBM_PEAK_GBS, 4)
     # what a plain device-to-device copy reaches on this box (1 GiB read + 1 GiB written), for orientation
     del idx, dist, nbr_sorted
     src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
