@@ -514,8 +514,20 @@ def cpu_reference_full(w, K, n):
         return {"value": None, "kind": "reference", "sample": "oracle/_ref is not built on this machine"}
     s = O.sorted_space(w["coords"], w["row_splits"], K)
     a = (s["scoords"], s["sbin"], s["sdbin"], s["bin_boundaries"], s["n_bins"], s["bin_width"], K)
+    import threading
+    done = threading.Event()
+
+    def heartbeat():            # minutes of silent CPU work: say so now and then
+        while not done.wait(30.0):
+            print("bench.py: reference CPU kernel still running (%.0f s)" % (time.perf_counter() - t0),
+                  file=sys.stderr, flush=True)
+
     t0 = time.perf_counter()
-    O.knn_sorted(*a, use_ref=True)
+    threading.Thread(target=heartbeat, daemon=True).start()
+    try:
+        O.knn_sorted(*a, use_ref=True)
+    finally:
+        done.set()
     t = time.perf_counter() - t0
     return {"value": round(n / t, 1), "unit": "queries/s", "cores": 1, "kind": "reference",
             "sample": "all %d queries of the bin-sorted workload, %.1f s, n_bins %s; kNN search kernel only"
