@@ -507,7 +507,7 @@ class _GravNetLayerCore(torch.autograd.Function):
         n, P = feat.shape
         dev = feat.device
         idx, dist, nbr_sorted, order = _knn_forward(coords, coords.shape[1], row_splits, K, None, None, 3, False,
-                                                    ctx.needs_input_grad[0])
+                                                    ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
         agg = torch.empty((n, 2 * P), dtype=torch.float32, device=dev)
         argmax = torch.empty((n, P), dtype=torch.int32, device=dev)
         if n > 0:
@@ -534,10 +534,17 @@ class _GravNetLayerCore(torch.autograd.Function):
             g_feat = torch.zeros_like(feat)
             g_dsq = torch.empty_like(dist)
             with torch.cuda.device(feat.device):
-                _lib.check(L.fgc_gravnet_aggregate_bwd_ld_f32(
-                    _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(feat), P, n, _lib.ptr(argmax), _lib.ptr(g_agg),
-                    ctypes.c_void_p(g_agg.data_ptr() + 4 * P), g_agg.stride(0), _lib.ptr(g_feat), P, _lib.ptr(g_dsq),
-                    n, K, P, None, _lib.stream_ptr()))
+                if config.tile_aggregation_backward and K <= 64 and 8 < P <= 64 and nbr_sorted.shape[0] == n:
+                    # rows that are neighbours in the search's sorted order share their targets: combined on chip
+                    _lib.check(L.fgc_gravnet_aggregate_bwd_sorted_f32(
+                        _lib.ptr(nbr_sorted), _lib.ptr(order), _lib.ptr(dist), _lib.ptr(feat), P, _lib.ptr(argmax),
+                        _lib.ptr(g_agg), ctypes.c_void_p(g_agg.data_ptr() + 4 * P), g_agg.stride(0), _lib.ptr(g_feat),
+                        P, _lib.ptr(g_dsq), n, K, P, None, _lib.stream_ptr()))
+                else:
+                    _lib.check(L.fgc_gravnet_aggregate_bwd_ld_f32(
+                        _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(feat), P, n, _lib.ptr(argmax), _lib.ptr(g_agg),
+                        ctypes.c_void_p(g_agg.data_ptr() + 4 * P), g_agg.stride(0), _lib.ptr(g_feat), P,
+                        _lib.ptr(g_dsq), n, K, P, None, _lib.stream_ptr()))
         if g_dist is not None:
             g_dsq = g_dist.to(torch.float32) if g_dsq is None else g_dsq + g_dist
         if ctx.needs_input_grad[0]:

@@ -763,8 +763,8 @@ __global__ __launch_bounds__(256) void k_gravnet_bwd(const int64_t *__restrict__
     // Slots are fetched PW at a time: lane j of the point's group reads slot kb + j (index, weight).  They are
     // then visited eight at a time: every lane takes its own feature(s) of the eight neighbours (gathers in
     // flight together), adds w * c to their feature gradients and keeps one partial dot product per slot; an
-    // exchange across the group's lanes (plain butterflies down to 8 lanes, then halving) leaves the dot
-    // product of slot j0 + (lane & 7) in every lane, and the lane that fetched that slot writes grad_distsq.
+    // exchange-halving across the group's lanes (fgc_group_reduce8) leaves the eight dot products spread over
+    // the group, and the lanes holding them write grad_distsq.
     bool bad = false;
     const bool single = P <= PW;      // one feature per lane: its upstream gradients stay in registers
     float cm0 = 0.f, gx0 = 0.f;
@@ -818,25 +818,212 @@ __global__ __launch_bounds__(256) void k_gravnet_bwd(const int64_t *__restrict__
                     }
                 }
             }
-#pragma unroll
-            for (int sft = PW / 2; sft >= 8; sft >>= 1) {
-#pragma unroll
-                for (int t = 0; t < 8; t++) vals[t] += __shfl_xor(vals[t], sft, 64);
-            }
-#pragma unroll
-            for (int sft = 4; sft >= 1; sft >>= 1) {
-                const bool upper = (pl & sft) != 0;
-#pragma unroll
-                for (int t = 0; t < sft; t++) {
-                    const float send = upper ? vals[t] : vals[t + sft];
-                    const float keep = upper ? vals[t + sft] : vals[t];
-                    vals[t] = keep + __shfl_xor(send, sft, 64);
-                }
-            }
-            if (qv && (pl & ~7) == j0 && kk < K) gdsq[i * K + kk] = -10.f * w_l * vals[0];
+            // the eight dot products, summed over the group's lanes by exchange-halving (DPP and lane swaps, no
+            // LDS permutes); the lane holds the total of slot j0 + ul and writes it with that slot's weight
+            const float tot = fgc_group_reduce8<PW>(vals, lane);
+            const int ul = pl * 8 / PW;
+            const float wu = __shfl(w_l, gbase + ((j0 + ul) & (PW - 1)), 64);
+            if (qv && (pl % (PW / 8)) == 0 && j0 + ul < cnt) gdsq[i * K + kb + j0 + ul] = -10.f * wu * tot;
         }
     }
     if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
+}
+
+// ---------------------------------------------------------------------------
+// The same backward for callers that have the neighbour rows in the search's sorted order (the fused GravNet
+// layer): the feature gradients of a tile of consecutive sorted rows are combined on chip before they go to memory.
+// ---------------------------------------------------------------------------
+// k_gravnet_bwd issues one atomic 128-byte row update per (point, slot) pair and is bound by the rate of those
+// updates.  Rows that are consecutive in the sorted order share most of their neighbours, so a wavefront (= one
+// block) here takes GT consecutive sorted rows and
+//   1. loads what the tile needs into LDS (per pair a record: target, weight; per row the upstream gradients and
+//      arg-max slots), then, per row pair with lane = feature, gathers the neighbours' feature rows and forms
+//      the dot products for grad_distsq as k_gravnet_bwd does - but does not touch grad_feat;
+//   2. groups the tile's records by target with a counting sort on the low bits of the target's sorted position
+//      (lane = record; LDS integer atomics for the ranks, one scan over the 1024 bucket counts);
+//   3. walks the grouped records with lane = feature (64 / PW records per instruction), recomputes each pair's
+//      contribution w * (g_mean / K + [argmax == slot] * g_max) from the rows kept in LDS, sums it in a register
+//      while the target stays the same, and issues ONE row update per run of equal targets.
+// For tiles of 8 (16) rows with K = 40 that is 2.1 (2.9) times fewer updates (sampled), and the result is the same
+// sum in another order.
+#ifndef GT
+#define GT 8             // sorted rows per wavefront (16: fewer row updates, but the longer serial walk of step 3 and
+#endif                   // half the wavefronts per CU cost more than they save: 1.15 against 0.84 ms at N=300k, K=40, P=32)
+#ifndef GT_BUCKETS
+#define GT_BUCKETS 512
+#endif
+
+template <int PW>
+__global__ __launch_bounds__(64) void k_gravnet_bwd_tile(const int *__restrict__ nbr, const uint32_t *__restrict__ order,
+                                                         const float *__restrict__ dsq, const float *__restrict__ feat,
+                                                         int ldf, const int *__restrict__ argmax,
+                                                         const float *__restrict__ gmean,
+                                                         const float *__restrict__ gmax, int ldg,
+                                                         float *__restrict__ gfeat, int ldgf,
+                                                         float *__restrict__ gdsq, int64_t n, int K, int P,
+                                                         int *__restrict__ status)
+{
+    constexpr int QPW = 64 / PW;               // rows per pass of step 1b, records per instruction of step 3
+    static_assert(GT % QPW == 0 && GT <= 64, "tile rows");
+    extern __shared__ __align__(16) unsigned char s_raw[];
+    const int lane = fgc_lane();
+    const int sub = lane / PW, pl = lane % PW;
+    // LDS: upstream rows [GT][PW] x 3, bucket counts, then the records: first as three arrays (target position,
+    // weight, target's original index) indexed [row][slot], later - over the same bytes - as 16-byte grouped records
+    float *rows_cm = (float *)s_raw;
+    float *rows_gx = rows_cm + GT * PW;
+    int *rows_am = (int *)(rows_gx + GT * PW);
+    int *hist = rows_am + GT * PW;
+    unsigned char *rec0 = (unsigned char *)(hist + GT_BUCKETS);
+    int *em = (int *)rec0;
+    float *ew = (float *)(em + GT * K);
+    int *eo = (int *)(ew + GT * K);
+    uint4 *srec = (uint4 *)rec0;
+    const int64_t r0 = (int64_t)blockIdx.x * GT;
+    const float invK = 1.0f / (float)K;
+    const unsigned ldf4 = 4u * (unsigned)ldf;
+    bool bad = false;
+    for (int t = lane; t < GT_BUCKETS; t += 64) hist[t] = 0;
+
+    // ---- 1a. everything the tile needs except the feature gathers, all loads independent of each other:
+    //      lane t keeps row t's original index; per row (lane = slot) the neighbour positions, their weights and
+    //      original indices go to LDS; per QPW rows (lane = feature) the upstream gradients and arg-max slots ----
+    const unsigned my_qo = (lane < GT && r0 + lane < n) ? order[r0 + lane] : 0u;
+#pragma unroll 4
+    for (int t = 0; t < GT; t++) {
+        const bool qv = r0 + t < n;
+        const int64_t qo = (int64_t)(unsigned)fgc_readlane_i((int)my_qo, t);
+        int m = -1, o = 0;
+        float w = 0.f;
+        if (qv && lane < K) {
+            m = nbr[(r0 + t) * K + lane];
+            w = expf(-10.f * dsq[qo * K + lane]);
+            if (m >= n) { bad = true; m = -1; }
+            if (m >= 0) o = (int)order[m];
+        }
+        if (lane < K) { em[t * K + lane] = m; ew[t * K + lane] = w; eo[t * K + lane] = o; }
+    }
+    for (int t0 = 0; t0 < GT; t0 += QPW) {
+        const int t = t0 + sub;
+        const bool qv = r0 + t < n;
+        const int64_t qo = (int64_t)(unsigned)__shfl((int)my_qo, t, 64);
+        float cm = 0.f, gx = 0.f;
+        int am = -1;
+        if (qv && pl < P) {
+            cm = gmean[qo * ldg + pl] * invK;
+            gx = gmax[qo * ldg + pl];
+            am = argmax[qo * P + pl];
+        }
+        rows_cm[t * PW + pl] = cm;
+        rows_gx[t * PW + pl] = gx;
+        rows_am[t * PW + pl] = am;
+    }
+
+    // ---- 1b. dot products for grad_distsq: lane = feature, QPW rows at a time, eight slots per step; the feature
+    //      gathers of the next step are requested before the current one is reduced ----
+    const int n_grp = (K + 7) >> 3;
+    for (int t0 = 0; t0 < GT; t0 += QPW) {
+        const int t = t0 + sub;
+        const bool qv = r0 + t < n;
+        const int64_t qo = (int64_t)(unsigned)__shfl((int)my_qo, t, 64);
+        const float cm = rows_cm[t * PW + pl], gx = rows_gx[t * PW + pl];
+        const int am = rows_am[t * PW + pl];
+        auto gather = [&](int g, float (&f)[8]) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int k = g * 8 + u;
+                f[u] = 0.f;
+                if (k < K && pl < P) {
+                    const int mu = em[t * K + k];
+                    if (mu >= 0) f[u] = *(const float *)((const char *)feat + (__umul24((unsigned)eo[t * K + k], ldf4) + 4u * (unsigned)pl));
+                }
+            }
+        };
+        float fcur[8], fnext[8];
+        gather(0, fcur);
+        for (int g = 0; g < n_grp; g++) {
+            if (g + 1 < n_grp) gather(g + 1, fnext);
+            float vals[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) vals[u] = fcur[u] * (cm + (am == g * 8 + u ? gx : 0.f));
+            const float tot = fgc_group_reduce8<PW>(vals, lane);
+            const int k = g * 8 + pl * 8 / PW;          // the slot whose total the lane holds
+            if (qv && (pl % (PW / 8)) == 0 && k < K) gdsq[qo * K + k] = -10.f * ew[t * K + k] * tot;
+#pragma unroll
+            for (int u = 0; u < 8; u++) fcur[u] = fnext[u];
+        }
+    }
+
+    // ---- 2. group the records by target: counting sort on the low bits of the target's sorted position ----
+    int rm[GT], ro[GT], rp[GT];
+    float rw[GT];
+#pragma unroll
+    for (int t = 0; t < GT; t++) {                    // lane = slot of row t
+        rm[t] = -1; ro[t] = 0; rp[t] = 0; rw[t] = 0.f;
+        if (lane < K) { rm[t] = em[t * K + lane]; rw[t] = ew[t * K + lane]; ro[t] = eo[t * K + lane]; }
+        if (rm[t] >= 0) rp[t] = atomicAdd(&hist[rm[t] & (GT_BUCKETS - 1)], 1);     // rank inside the bucket
+    }
+    asm volatile("" ::: "memory");     // the records are read before anything is written over them (other types below)
+    // exclusive scan of the bucket counts: consecutive buckets per lane, then across the lanes
+    int cntv[GT_BUCKETS / 64], run = 0;
+#pragma unroll
+    for (int b = 0; b < GT_BUCKETS / 64; b++) { cntv[b] = hist[lane * (GT_BUCKETS / 64) + b]; run += cntv[b]; }
+    int incl = run;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+    }
+    const int n_rec = __shfl(incl, 63, 64);
+    int base = incl - run;
+#pragma unroll
+    for (int b = 0; b < GT_BUCKETS / 64; b++) { hist[lane * (GT_BUCKETS / 64) + b] = base; base += cntv[b]; }
+    // every record is in registers by now: the grouped records may overwrite the three arrays
+#pragma unroll
+    for (int t = 0; t < GT; t++) {
+        if (rm[t] >= 0) {
+            const int dst = hist[rm[t] & (GT_BUCKETS - 1)] + rp[t];
+            srec[dst] = make_uint4((unsigned)ro[t], __float_as_uint(rw[t]), (unsigned)((t << 8) | lane), (unsigned)rm[t]);
+        }
+    }
+
+    // ---- 3. one row update per run of equal targets; lane = feature, QPW records per instruction ----
+    const int per = (n_rec + QPW - 1) / QPW;
+    const int j_beg = sub * per, j_end = min(n_rec, j_beg + per);
+    int cur = -1;
+    float acc = 0.f;
+    for (int j = j_beg; j < j_beg + per; j += 4) {
+        uint4 rc[4];
+        float cmv[4], gxv[4];
+        int amv[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            rc[u] = (j + u < j_end) ? srec[j + u] : make_uint4(0xffffffffu, 0u, 0u, 0u);
+            const int t = (int)(rc[u].z >> 8) & (GT - 1);
+            cmv[u] = rows_cm[t * PW + pl];
+            gxv[u] = rows_gx[t * PW + pl];
+            amv[u] = rows_am[t * PW + pl];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int tgt = (int)rc[u].x;
+            if (j + u < j_end) {
+                if (tgt != cur) {
+                    if (cur >= 0 && cur < n && pl < P) atomicAdd(&gfeat[(int64_t)cur * ldgf + pl], acc);
+                    cur = tgt;
+                    acc = 0.f;
+                }
+                acc += __uint_as_float(rc[u].y) * (cmv[u] + (amv[u] == (int)(rc[u].z & 255u) ? gxv[u] : 0.f));
+            }
+        }
+    }
+    if (cur >= 0 && cur < n && pl < P) atomicAdd(&gfeat[(int64_t)cur * ldgf + pl], acc);
+    if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
+}
+
+static size_t gravnet_tile_lds(int pw, int K)
+{
+    return (size_t)GT * pw * 12 + (size_t)GT_BUCKETS * 4 + (size_t)GT * K * 16;
 }
 
 static int pick_pw(int P)
@@ -907,6 +1094,41 @@ extern "C" int fgc_gravnet_aggregate_bwd_ld_f32(const int64_t *d_idx, const floa
                        (int)ld_grad_feat, d_grad_distsq, n_vert, (int)K, (int)P, d_status)
     switch (pw) {
     case 8: FGC_L(8); break;
+    case 16: FGC_L(16); break;
+    case 32: FGC_L(32); break;
+    default: FGC_L(64); break;
+    }
+#undef FGC_L
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
+}
+
+extern "C" int fgc_gravnet_aggregate_bwd_sorted_f32(const int32_t *d_nbr_sorted, const int32_t *d_order,
+                                                    const float *d_distsq, const float *d_feat, int32_t ld_feat,
+                                                    const int32_t *d_argmax, const float *d_grad_fmean,
+                                                    const float *d_grad_fmax, int32_t ld_grad, float *d_grad_feat,
+                                                    int32_t ld_grad_feat, float *d_grad_distsq, int64_t n_vert,
+                                                    int32_t K, int32_t P, int32_t *d_status, void *stream)
+{
+    if (n_vert < 0 || K < 1 || P < 1 || ld_feat < P || ld_grad < P || ld_grad_feat < P) return FGC_EINVAL;
+    if (K > 64 || P > 64 || P <= 8 || n_vert >= (1ll << 31) - 1) return FGC_EUNSUPPORTED;
+    // 32-bit byte offsets of the feature rows, formed with a 24-bit multiply
+    if (n_vert >= (1 << 24) || ld_feat >= (1 << 22) || (uint64_t)n_vert * (uint64_t)ld_feat * 4ull >= 0xffffffffull)
+        return FGC_EUNSUPPORTED;
+    if (n_vert == 0) return FGC_OK;
+    if (!d_nbr_sorted || !d_order || !d_distsq || !d_feat || !d_argmax || !d_grad_fmean || !d_grad_fmax ||
+        !d_grad_feat || !d_grad_distsq)
+        return FGC_EINVAL;
+    hipStream_t s = (hipStream_t)stream;
+    const int pw = pick_pw(P);
+    const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GT);
+    const size_t lds = gravnet_tile_lds(pw, K);
+#define FGC_L(PWW)                                                                                              \
+    hipLaunchKernelGGL((k_gravnet_bwd_tile<PWW>), dim3(blocks), dim3(64), lds, s, d_nbr_sorted,                \
+                       (const uint32_t *)d_order, d_distsq, d_feat, (int)ld_feat, d_argmax, d_grad_fmean,      \
+                       d_grad_fmax, (int)ld_grad, d_grad_feat, (int)ld_grad_feat, d_grad_distsq, n_vert, (int)K, \
+                       (int)P, d_status)
+    switch (pw) {
     case 16: FGC_L(16); break;
     case 32: FGC_L(32); break;
     default: FGC_L(64); break;

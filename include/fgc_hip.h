@@ -301,6 +301,18 @@ int fgc_gravnet_aggregate_bwd_ld_f32(const int64_t *d_idx, const float *d_distsq
                                      float *d_grad_feat, int32_t ld_grad_feat, float *d_grad_distsq,
                                      int64_t n_vert, int32_t K, int32_t P, int32_t *d_status, void *stream);
 
+/* The backward for callers that hold the neighbour rows in the search's sorted order (d_nbr_sorted and d_order as
+ * for fgc_binned_select_knn_grad_sorted_f32; everything else - d_distsq, d_feat, d_argmax, the gradients - stays in
+ * the original order): the feature gradients of 16 consecutive sorted rows, which share most of their neighbours,
+ * are combined on chip, so that one row update per distinct target of the tile reaches memory instead of one per
+ * (point, slot) pair.  Same results as fgc_gravnet_aggregate_bwd_ld_f32 up to the order of the float sums.
+ * Supports K <= 64 and 8 < P <= 64 (FGC_EUNSUPPORTED otherwise: use the entry point above). */
+int fgc_gravnet_aggregate_bwd_sorted_f32(const int32_t *d_nbr_sorted, const int32_t *d_order, const float *d_distsq,
+                                         const float *d_feat, int32_t ld_feat, const int32_t *d_argmax,
+                                         const float *d_grad_fmean, const float *d_grad_fmax, int32_t ld_grad,
+                                         float *d_grad_feat, int32_t ld_grad_feat, float *d_grad_distsq,
+                                         int64_t n_vert, int32_t K, int32_t P, int32_t *d_status, void *stream);
+
 /* ---------------------------------------------------------------------------
  * Weight and bias gradient of a dense layer y = x W^T + b over n points:
  *   d_grad_weight [n_out, n_in] = grad_out^T x,  d_grad_bias [n_out] = column sums

@@ -346,3 +346,64 @@ def test_gravnet_aggregate_closed_forms():
                              torch.from_numpy(f).cuda())
     np.testing.assert_array_equal(m.cpu().numpy(), f)
     np.testing.assert_array_equal(x.cpu().numpy(), f)
+
+
+@pytest.mark.parametrize("n,S,K,P,events", [(5000, 4, 40, 32, 2), (3001, 3, 64, 64, 3), (4000, 2, 7, 20, 1),
+                                            (2500, 5, 24, 16, 4), (777, 4, 33, 9, 2)])
+def test_gravnet_backward_in_sorted_space(oracle, n, S, K, P, events):
+    """fgc_gravnet_aggregate_bwd_sorted_f32 (feature gradients of a tile of sorted rows combined on chip) through the
+    C ABI against the per-pair kernel and against autograd through the checker's torch composition; padding (events
+    smaller than K) included."""
+    import ctypes
+    from fastgraphcompute_amd import _lib, _ops
+    L = _lib.lib()
+    rng = np.random.default_rng(n + K + P)
+    space = torch.from_numpy((rng.standard_normal((n, S)) * 0.2).astype(np.float32)).cuda()
+    cuts = sorted(rng.choice(np.arange(1, n), events - 1, replace=False).tolist()) if events > 1 else []
+    if events > 2:
+        cuts[0] = min(cuts[0], K // 2)                      # a first event smaller than K: padded rows
+    rs = torch.tensor([0] + sorted(cuts) + [n], device="cuda")
+    idx, dist, nbr, order = _ops._knn_forward(space, S, rs, K, None, None, 3, False, True)
+    feat = torch.from_numpy(rng.standard_normal((n, P)).astype(np.float32)).cuda()
+    fm = torch.empty((n, P), device="cuda")
+    fx = torch.empty((n, P), device="cuda")
+    am = torch.empty((n, P), dtype=torch.int32, device="cuda")
+    st = _lib.stream_ptr()
+    _lib.check(L.fgc_gravnet_aggregate_fwd_f32(_lib.ptr(idx), _lib.ptr(dist), _lib.ptr(feat), _lib.ptr(fm), _lib.ptr(fx),
+                                               _lib.ptr(am), n, K, P, st))
+    g = torch.from_numpy(rng.standard_normal((n, 2 * P)).astype(np.float32)).cuda()     # (d mean | d max) side by side
+    out = {}
+    for name in ("pairs", "tiles"):
+        gf = torch.zeros((n, P), device="cuda")
+        gd = torch.full((n, K), 7.0, device="cuda")
+        if name == "pairs":
+            rc = L.fgc_gravnet_aggregate_bwd_ld_f32(_lib.ptr(idx), _lib.ptr(dist), _lib.ptr(feat), P, n, _lib.ptr(am),
+                                                    _lib.ptr(g), ctypes.c_void_p(g.data_ptr() + 4 * P), 2 * P,
+                                                    _lib.ptr(gf), P, _lib.ptr(gd), n, K, P, None, st)
+        else:
+            rc = L.fgc_gravnet_aggregate_bwd_sorted_f32(_lib.ptr(nbr), _lib.ptr(order), _lib.ptr(dist), _lib.ptr(feat),
+                                                        P, _lib.ptr(am), _lib.ptr(g),
+                                                        ctypes.c_void_p(g.data_ptr() + 4 * P), 2 * P, _lib.ptr(gf), P,
+                                                        _lib.ptr(gd), n, K, P, None, st)
+        _lib.check(rc)
+        torch.cuda.synchronize()
+        out[name] = (gf.cpu().numpy(), gd.cpu().numpy())
+    assert _rel_err(out["tiles"][0], out["pairs"][0]) < DIST_RTOL
+    np.testing.assert_array_equal(out["tiles"][1], out["pairs"][1])          # same operations in the same order
+    # against autograd through the torch composition of the reference's aggregation
+    it, dt, ft = idx.cpu(), dist.cpu().requires_grad_(True), feat.cpu().requires_grad_(True)
+    tm, tx = oracle.gravnet_aggregate_torch(it, dt, ft)
+    ((tm * g[:, :P].cpu()).sum() + (tx * g[:, P:].cpu()).sum()).backward()
+    assert _rel_err(out["tiles"][0], ft.grad.numpy()) < DIST_RTOL
+    assert _rel_err(out["tiles"][1], dt.grad.numpy()) < DIST_RTOL
+
+
+def test_gravnet_backward_in_sorted_space_rejects_unsupported_shapes():
+    from fastgraphcompute_amd import _lib
+    L = _lib.lib()
+    fake = ctypes_ptr = None
+    import ctypes
+    p = ctypes.c_void_p(4096)
+    assert L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, 32, p, p, p, 32, p, 32, p, 100, 65, 32, None, None) == -3
+    assert L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, 8, p, p, p, 8, p, 8, p, 100, 8, 8, None, None) == -3
+    assert L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, 16, p, p, p, 32, p, 32, p, 100, 8, 32, None, None) == -1
