@@ -317,8 +317,8 @@ def gravnet_stage_times(op, x, rs, w, dev):
     with torch.no_grad():
         space = op.space_transformations(x).contiguous()
         feat = op.propagate_transformations(x).contiguous()
-    import fastgraphcompute_amd as fgc
-    idx, dist = fgc.binned_select_knn(int(w["K"]), space, rs)
+    from fastgraphcompute_amd import _ops
+    idx, dist, nbr_sorted, order = _ops._knn_forward(space, space.shape[1], rs, int(w["K"]), None, None, 3, False, True)
     n, K = idx.shape
     P = feat.shape[1]
     agg = torch.empty((n, 2 * P), device=dev)
@@ -333,10 +333,16 @@ def gravnet_stage_times(op, x, rs, w, dev):
                                                       ctypes.c_void_p(agg.data_ptr() + 4 * P), 2 * P, _lib.ptr(am), n,
                                                       K, P, None, st))
 
-    def bwd():
+    def bwd_pairs():     # one atomic row update per (point, slot) pair: the stand-alone op's kernel
         _lib.check(L.fgc_gravnet_aggregate_bwd_ld_f32(_lib.ptr(idx), _lib.ptr(dist), _lib.ptr(feat), P, n, _lib.ptr(am),
                                                       _lib.ptr(g_agg), ctypes.c_void_p(g_agg.data_ptr() + 4 * P),
                                                       2 * P, _lib.ptr(g_feat), P, _lib.ptr(g_dsq), n, K, P, None, st))
+
+    def bwd():           # what GravNetOp's backward runs: rows of a sorted tile combined on chip
+        _lib.check(L.fgc_gravnet_aggregate_bwd_sorted_f32(_lib.ptr(nbr_sorted), _lib.ptr(order), _lib.ptr(dist),
+                                                          _lib.ptr(feat), P, _lib.ptr(am), _lib.ptr(g_agg),
+                                                          ctypes.c_void_p(g_agg.data_ptr() + 4 * P), 2 * P,
+                                                          _lib.ptr(g_feat), P, _lib.ptr(g_dsq), n, K, P, None, st))
 
     def timed(fn, reps=8):
         ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
@@ -347,14 +353,19 @@ def gravnet_stage_times(op, x, rs, w, dev):
         torch.cuda.synchronize()
         return float(np.median([a.elapsed_time(b) for a, b in ev][2:]))
 
-    t_fwd, t_bwd = timed(fwd), timed(bwd)
+    fwd()                # the backward kernels read the arg-max slots the forward writes
+    tiled = K <= 64 and 8 < P <= 64
+    t_fwd, t_bwd_pairs = timed(fwd), timed(bwd_pairs)
+    t_bwd = timed(bwd) if tiled else t_bwd_pairs
     clock_hz = GPU_CLOCK_HZ
     facts = profile_facts()
     # index + distance rows, one P-float gather per pair, features / outputs once; the backward gathers and scatters
     fwd_alg = 12.0 * K * n + 4.0 * P * n * K + 8.0 * P * n
     bwd_alg = fwd_alg + 4.0 * P * n * K
-    return {"stages_ms": {"aggregate_fwd": round(t_fwd, 4), "aggregate_bwd": round(t_bwd, 4)},
-            "roofline": roofline_entry("k_gravnet_bwd", w["name"], bwd_alg, t_bwd, clock_hz, None, facts),
+    return {"stages_ms": {"aggregate_fwd": round(t_fwd, 4), "aggregate_bwd": round(t_bwd, 4),
+                          "aggregate_bwd_per_pair_kernel": round(t_bwd_pairs, 4)},
+            "roofline": roofline_entry("k_gravnet_bwd_tile" if tiled else "k_gravnet_bwd", w["name"], bwd_alg, t_bwd,
+                                       clock_hz, None, facts),
             "roofline_aggregate_fwd": roofline_entry("k_gravnet_fwd", w["name"], fwd_alg, t_fwd, clock_hz, None, facts)}
 
 
