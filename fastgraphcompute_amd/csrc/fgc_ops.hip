@@ -291,8 +291,8 @@ __global__ __launch_bounds__(256) void k_sorted_points(const float *__restrict__
 #define GSH 512      // table slots per wavefront where an entry is 16 bytes (D <= 3)
 #endif
 #ifndef GSW
-#define GSW 32       // queries per wavefront where an entry is 16 bytes
-#endif
+#define GSW 24       // rows per wavefront where an entry is 16 bytes (N=1M, D=3, K=64: 16 rows 0.53 ms, 20 0.44, 24 0.43,
+#endif               // 32 0.47, 48 0.49: fewer rows share less, more rows fill the table and wait longer for their loads)
 
 // Totals of 16 per-lane values over the 64 lanes, in 36 instead of 16 x 11 instructions: each exchange step
 // halves the number of values a lane still carries (the lane keeps the half its own bit selects and hands the
