@@ -89,6 +89,9 @@ def main():
     ap.add_argument("--cpu-reference-full", action="store_true",
                     help="also time the reference's own compiled CPU kernel (oracle/_ref) on ALL queries of the "
                          "workload, one core; minutes at the default workload")
+    ap.add_argument("--sorted-neighbours", action="store_true",
+                    help="ask for neighbour rows by increasing distance (config.sorted_neighbours) instead of the "
+                         "default, rows in the order the search found them, as the reference returns them")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no multi-GPU part); "
@@ -109,6 +112,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     L = _lib.lib()
+    config.sorted_neighbours = bool(args.sorted_neighbours)
 
     if args.workload == "oc_helper":
         print(json.dumps(oc_helper_workload(args, dev)), flush=True)
@@ -168,13 +172,14 @@ def main():
     dist = torch.empty((n, K), dtype=torch.float32, device=dev)
     nbr_sorted = torch.empty((n, K), dtype=torch.int32, device=dev)   # as the autograd path requests it
     st = _lib.stream_ptr()
+    knn_flags = 0 if config.sorted_neighbours else _lib.KNN_ANY_ORDER     # the row order binned_select_knn asks for
 
     def prepare():
         _lib.check(L.fgc_binned_knn_prepare_f32(_lib.ptr(coords), n, D, _lib.ptr(rs), rs_arr, n_rs, K, nbd, nb_arr,
                                                 None, _lib.ptr(status), _lib.ptr(ws), ws_bytes, st))
 
     def search(with_stats):
-        _lib.check(L.fgc_binned_knn_search_f32(n, D, rs_arr, n_rs, K, nbd, nb_arr, 0, 0, _lib.ptr(idx), _lib.ptr(dist),
+        _lib.check(L.fgc_binned_knn_search_f32(n, D, rs_arr, n_rs, K, nbd, nb_arr, 0, knn_flags, _lib.ptr(idx), _lib.ptr(dist),
                                                _lib.ptr(nbr_sorted),
                                                _lib.ptr(stats) if with_stats else None, _lib.ptr(ws), ws_bytes, st))
 
@@ -239,7 +244,8 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(t_step * 1e3, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": w["name"], "n_points": n, "n_coords": D, "K": K, "events": int(n_rs - 1),
-                   "n_bins": nb, "step": "binned_select_knn forward (whole call) + gradient"},
+                   "n_bins": nb, "step": "binned_select_knn forward (whole call) + gradient",
+                   "row_order": "by distance" if config.sorted_neighbours else "any (as the reference)"},
         "neighbours_per_s": round(n * K / t_step, 1),
         "forward_call_ms": round(t_prep + t_knn, 4),
         "forward_queries_per_s": round(n / ((t_prep + t_knn) * 1e-3), 1),

@@ -308,7 +308,8 @@ def _knn_forward(coords: torch.Tensor, D: int, row_splits, K: int, direction, n_
                 # (int32) and the permutation
                 nbr_sorted = torch.empty((n, K), dtype=torch.int32, device=dev)
             _lib.check(L.fgc_binned_knn_search_f32(
-                n, D, rs_arr, n_rs, K, nbd, nb_arr, 1 if dirt is not None else 0, 1 if tf_compat else 0,
+                n, D, rs_arr, n_rs, K, nbd, nb_arr, 1 if dirt is not None else 0,
+                (_lib.KNN_TF_COMPAT if tf_compat else 0) | (0 if config.sorted_neighbours else _lib.KNN_ANY_ORDER),
                 _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(nbr_sorted), _lib.ptr(stats), _lib.ptr(ws), ws_bytes, st))
             if want_backward:
                 order = torch.empty(n, dtype=torch.int32, device=dev)

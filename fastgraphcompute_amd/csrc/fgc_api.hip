@@ -210,7 +210,8 @@ int knn_search(float tau0, int32_t *d_nbr_sorted, int64_t n_vert, int32_t n_coor
     a.n_super = (a.n_chunks + 63) / 64;
     a.bb = (const int *)(ws + c.w.bb); a.geom = (const float *)(ws + c.w.geom);
     a.sdir = with_direction ? (const unsigned char *)(ws + c.w.sdir) : nullptr;
-    a.n = (int)n_vert; a.D = n_coords; a.nbd = n_bin_dims; a.K = K; a.tf_compat = tf_compat;
+    a.n = (int)n_vert; a.D = n_coords; a.nbd = n_bin_dims; a.K = K;
+    a.tf_compat = (tf_compat & FGC_KNN_TF_COMPAT) != 0; a.any_order = (tf_compat & FGC_KNN_ANY_ORDER) != 0;
     a.tau0 = tau0;
     a.out_sorted = d_nbr_sorted;
     a.out_idx = d_idx; a.out_dist = d_distsq; a.stats = (unsigned long long *)d_stats;

@@ -33,7 +33,8 @@ struct KnnArgs {
     int D;                      // coordinates per point
     int nbd;                    // binned dimensions
     int K;
-    int tf_compat;
+    int tf_compat;              // padding slots name the query itself instead of -1
+    int any_order;              // rows may be written in pool order (slot 0 still the query itself) instead of by distance
     float tau0;                 // initial bound on the squared neighbour distance (INFINITY: none); exclusive
     int pool_cap;               // candidate pool slots per query (set by fgc_launch_knn)
     int64_t *out_idx;           // [n, K] original order

@@ -16,7 +16,8 @@
 // bisection on the distance threshold, counted with wave ballots over the pool
 // held one slot per lane, finds a tighter tau and the survivors are compacted.
 // The steady-state loop is subtract / multiply / add / compare; exact selection
-// of the K best and the sort by distance happen once per query at the end.
+// of the K best happens once per query at the end, followed by a sort by distance
+// only when the caller asks for ordered rows (the reference's rows have no order).
 //
 // Search order for the queries of a wavefront that share a bin row (all binned
 // coordinates but the last one):
@@ -657,6 +658,40 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
         const long long orig_q = (long long)a.order[self];
         // the sort below takes NSEG * 64 entries: a pool that fits is sorted as it is and its first K entries are
         // written, a larger one is first cut to exactly K
+        if (a.any_order) {
+            // Rows in pool order: cut the pool to exactly K, move the query itself to slot 0 (its entry trades places
+            // with the one in slot 0) and write - no sort.  A pool without the query (direction flags, or more than K
+            // points at distance 0) takes the sorting path below, which drops the farthest entry for it.
+            if (fgc_readlane_i(cnt, q) > K) prune(q, true);
+            const int c = fgc_readlane_i(cnt, q);
+            int es = -1;                          // element that holds the query
+            unsigned EX[NSEG], EY[NSEG];
+#pragma unroll
+            for (int s = 0; s < NSEG; s++) {
+                const bool valid = (s * 64 + lane) < c;
+                const uint2 e = valid ? pool[q * CAP + s * 64 + lane] : make_uint2(0x7f800000u, 0xffffffffu);
+                EX[s] = e.x; EY[s] = e.y;
+                const unsigned long long sm = fgc_ballot(valid && (int)e.y == self);
+                if (sm) es = s * 64 + __ffsll((long long)sm) - 1;
+            }
+            if (es >= 0) {
+#pragma unroll
+                for (int s = 0; s < NSEG; s++) {
+                    const int e = s * 64 + lane;
+                    if (e < c) {
+                        const int slot = e == es ? 0 : (e == 0 ? es : e);
+                        a.out_idx[orig_q * K + slot] = e == es ? orig_q : (long long)a.order[EY[s]];
+                        a.out_dist[orig_q * K + slot] = e == es ? 0.f : __uint_as_float(EX[s]);
+                        if (a.out_sorted) a.out_sorted[(long long)self * K + slot] = (int)EY[s];
+                    } else if (e < K) {
+                        a.out_idx[orig_q * K + e] = a.tf_compat ? orig_q : -1ll;
+                        a.out_dist[orig_q * K + e] = 0.f;
+                        if (a.out_sorted) a.out_sorted[(long long)self * K + e] = -1;
+                    }
+                }
+                continue;
+            }
+        }
         if (fgc_readlane_i(cnt, q) > NSEG * 64) prune(q, true);
         const int c = fgc_readlane_i(cnt, q);     // entries in slots 0..c-1, c <= NSEG * 64
         float L[NSEG];

@@ -26,8 +26,10 @@ def binned_select_knn(K: int,
     """Exact K nearest neighbours of every point inside its own event.
 
     Returns (idx int64 [N, K], distsq float32 [N, K]); column 0 is the point
-    itself with distance 0, the other columns its K-1 nearest neighbours (by
-    increasing distance), -1 / 0 where the event has fewer than K points.
+    itself with distance 0, the other columns its K-1 nearest neighbours, then
+    -1 / 0 where the event has fewer than K points.  Like the reference, the
+    neighbours of a row come in no particular order; set
+    config.sorted_neighbours for rows by increasing distance.
     `direction`: 0 = may only be a neighbour, 1 = may only have neighbours, 2 = neither.
     """
     if coords.dim() != 2 or coords.shape[1] == 0:

@@ -38,6 +38,13 @@ extern "C" {
 #define FGC_MAX_K 1024       /* neighbours per query the kNN kernels support; the reference's loops take any
                                 K (binned_select_knn_cpu.cpp:211-326), its benchmarks stop at 100.  Up to 256
                                 the search runs its register-tiled kernels, beyond that a slower variant  */
+/* bits of the kNN entry points' tf_compat argument */
+#define FGC_KNN_TF_COMPAT 1  /* padding slots name the query itself instead of -1 (binned_select_knn.py:7-9) */
+#define FGC_KNN_ANY_ORDER 2  /* slots 1.. of a row in any order instead of by increasing distance: the reference
+                                promises no order either (its kernel replaces the farthest entry in place, its tests
+                                sort every row before comparing, tests/test_binned_select_knn.py:90-91); saves the
+                                per-query sort */
+
 #define FGC_STATUS_WORDS 4
 /* bits of d_status[0] */
 #define FGC_ST_NONFINITE 1   /* a binned coordinate is inf/nan                */
@@ -110,9 +117,11 @@ int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t ld_coords,
  *                 :67-82) or passes the user's n_bins
  *   d_direction   int64 [n_vert] or NULL (0: only neighbour, 1: only query,
  *                 2: neither; binned_select_knn_cuda_kernel.cu:120-122,194-196)
+ *   tf_compat     bit set of FGC_KNN_TF_COMPAT and FGC_KNN_ANY_ORDER (0 or 1 as before: rows by distance)
  *   d_idx         out int64 [n_vert, K]: slot 0 the query itself, then its
- *                 K-1 nearest points of the same event by increasing distance,
- *                 -1 (or the query's index if tf_compat) where the event has
+ *                 K-1 nearest points of the same event by increasing distance
+ *                 (in any order with FGC_KNN_ANY_ORDER), then -1 (or the
+ *                 query's index with FGC_KNN_TF_COMPAT) where the event has
  *                 fewer than K points
  *   d_distsq      out float32 [n_vert, K], 0 for slot 0 and for padding
  *   d_stats       optional uint64[8] device counters, accumulated: [0] distance

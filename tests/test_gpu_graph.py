@@ -26,7 +26,8 @@ def test_forward_captured_in_a_graph_replays_correctly():
     dist = torch.empty((n, K), dtype=torch.float32, device="cuda")
 
     def enqueue():
-        _lib.check(L.fgc_binned_select_knn_f32(_lib.ptr(coords), n, D, _lib.ptr(rs), rsa, 3, K, nbd, nb, None, 0,
+        _lib.check(L.fgc_binned_select_knn_f32(_lib.ptr(coords), n, D, _lib.ptr(rs), rsa, 3, K, nbd, nb, None,
+                                               _lib.KNN_ANY_ORDER,       # the row order binned_select_knn asks for
                                                _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(status), None, _lib.ptr(ws),
                                                ws_bytes, _lib.stream_ptr()))
 

@@ -21,6 +21,12 @@ def _gpu_knn(K, coords, rs, **kw):
     return idx.cpu().numpy(), dist.cpu().numpy()
 
 
+def _padding_last(idx):
+    """Empty slots (-1) only after the last neighbour of a row."""
+    empty = idx < 0
+    assert not np.any(empty[:, :-1] & ~empty[:, 1:]), "a neighbour after an empty slot"
+
+
 def _check(oracle, K, coords, rs, threads=8, **kw):
     """GPU result against the checker - with the library's own search grid and, when the caller gives no n_bins,
     also with the reference's grid (its n_bins heuristic and max_bin_dims)."""
@@ -29,6 +35,21 @@ def _check(oracle, K, coords, rs, threads=8, **kw):
     okw = {k: (v.cpu().numpy() if torch.is_tensor(v) else v) for k, v in kw.items()}
     oi, od = oracle.binned_select_knn(K, coords, rs, n_threads=threads, **okw)
     assert_knn_equal(gi, gd, oi, od, what="own grid")
+    _padding_last(gi)
+    # the same call with rows by increasing distance (config.sorted_neighbours; the default leaves slots 1.. in the
+    # order the search found them, like the reference)
+    config.sorted_neighbours = True
+    try:
+        si, sd = _gpu_knn(K, coords, rs, **dict(kw))
+    finally:
+        config.sorted_neighbours = False
+    assert_knn_equal(si, sd, oi, od, what="rows by distance")
+    _padding_last(si)
+    if not kw.get("torch_compatible_indices"):
+        filled = np.where(si[:, 1:] >= 0, sd[:, 1:], np.inf)
+        with np.errstate(invalid="ignore"):
+            step = np.diff(filled, axis=1)                      # inf - inf between two empty slots
+        assert np.all((step >= 0) | np.isnan(step)), "rows not ascending with config.sorted_neighbours"
     if kw.get("n_bins") is None:
         config.auto_grid = False
         try:
@@ -135,9 +156,7 @@ def test_small_and_empty_events(oracle):
     gi, gd = _check(oracle, 20, coords, rs)
     check_knn_properties(gi, gd, coords, rs, 20)
     assert (gi[:3, 3:] == -1).all() and (gd[:3, 3:] == 0).all()
-    ti, td = _gpu_knn(20, coords, rs, torch_compatible_indices=True)
-    oi, od = oracle.binned_select_knn(20, coords, rs, torch_compatible_indices=True)
-    assert_knn_equal(ti, td, oi, od)
+    ti, td = _check(oracle, 20, coords, rs, torch_compatible_indices=True)
     assert (ti[:3, 3:] == np.arange(3)[:, None]).all()
 
 

@@ -129,7 +129,7 @@ def test_knn_threads_and_sampling_agree(oracle):
     np.testing.assert_array_equal(i1, i8)
     np.testing.assert_array_equal(d1, d8)
     assert st1["C_eval"] == st8["C_eval"]
-    check_knn_properties(*_sorted_rows(i1, d1), w["coords"], w["row_splits"], w["K"])
+    check_knn_properties(*_sorted_rows(i1, d1), w["coords"], w["row_splits"], w["K"], ascending=True)
 
 
 def _sorted_rows(idx, dist):

@@ -47,8 +47,9 @@ def assert_knn_equal(idx_a, dist_a, idx_b, dist_b, what=""):
                 np.testing.assert_allclose(da[r, cols], db[r, cols], rtol=TIE_RTOL, atol=0)
 
 
-def check_knn_properties(idx, dist, coords, row_splits, K):
-    """Size-independent invariants of a kNN result (used at full benchmark sizes)."""
+def check_knn_properties(idx, dist, coords, row_splits, K, ascending=False):
+    """Size-independent invariants of a kNN result (used at full benchmark sizes).  ascending: the rows were asked
+    for by increasing distance (config.sorted_neighbours, or rows sorted by the caller)."""
     idx = np.asarray(idx)
     dist = np.asarray(dist)
     n = coords.shape[0]
@@ -63,11 +64,14 @@ def check_knn_properties(idx, dist, coords, row_splits, K):
     sizes = np.diff(np.asarray(row_splits))[ev]
     np.testing.assert_array_equal(valid.sum(axis=1), np.minimum(sizes, K))
     assert np.all(dist[~valid] == 0)
-    # slots 1.. ascending in distance over the valid part
-    d = np.where(valid, dist, np.inf)
-    with np.errstate(invalid="ignore"):
-        dd = np.diff(d[:, 1:], axis=1)
-    assert np.all((dd >= 0) | np.isnan(dd)), "row not sorted by distance"
+    # empty slots only at the end of a row
+    assert not np.any(~valid[:, :-1] & valid[:, 1:]), "a neighbour after an empty slot"
+    if ascending:
+        # slots 1.. ascending in distance over the valid part
+        d = np.where(valid, dist, np.inf)
+        with np.errstate(invalid="ignore"):
+            dd = np.diff(d[:, 1:], axis=1)
+        assert np.all((dd >= 0) | np.isnan(dd)), "row not sorted by distance"
     # no duplicate neighbours in a row
     s = np.sort(np.where(valid, idx, -np.arange(1, K + 1)[None, :]), axis=1)
     assert np.all(np.diff(s, axis=1) != 0), "duplicate neighbour"
