@@ -1,5 +1,6 @@
 // index_replacer, kNN gradient, select_with_default and the fused GravNet
 // neighbour aggregation (forward / backward).  gfx950, wave64.
+#include <atomic>
 #include "fgc_common.h"
 #include "fgc_internal.h"
 
@@ -834,62 +835,78 @@ __global__ __launch_bounds__(256) void k_gravnet_bwd(const int64_t *__restrict__
 // layer): the feature gradients of a tile of consecutive sorted rows are combined on chip before they go to memory.
 // ---------------------------------------------------------------------------
 // k_gravnet_bwd issues one atomic 128-byte row update per (point, slot) pair and is bound by the rate of those
-// updates.  Rows that are consecutive in the sorted order share most of their neighbours, so a wavefront (= one
-// block) here takes GT consecutive sorted rows and
-//   1. loads what the tile needs into LDS (per pair a record: target, weight; per row the upstream gradients and
-//      arg-max slots), then, per row pair with lane = feature, gathers the neighbours' feature rows and forms
-//      the dot products for grad_distsq as k_gravnet_bwd does - but does not touch grad_feat;
-//   2. groups the tile's records by target with a counting sort on the low bits of the target's sorted position
-//      (lane = record; LDS integer atomics for the ranks, one scan over the 1024 bucket counts);
-//   3. walks the grouped records with lane = feature (64 / PW records per instruction), recomputes each pair's
-//      contribution w * (g_mean / K + [argmax == slot] * g_max) from the rows kept in LDS, sums it in a register
-//      while the target stays the same, and issues ONE row update per run of equal targets.
-// For tiles of 8 (16) rows with K = 40 that is 2.1 (2.9) times fewer updates (sampled), and the result is the same
-// sum in another order.
+// updates.  Rows that are consecutive in the sorted order share most of their neighbours, so a block of GT_WAVES
+// wavefronts here takes GT_WAVES * GT consecutive sorted rows and
+//   1. each wavefront loads what its GT rows need into LDS (per pair a record: target, weight; per row the upstream
+//      gradients and arg-max slots), then, per row pair with lane = feature, gathers the neighbours' feature rows
+//      and forms the dot products for grad_distsq as k_gravnet_bwd does - but does not touch grad_feat;
+//   2. the block groups all its records by target with a counting sort on the low bits of the target's sorted
+//      position (lane = record; LDS integer atomics for the ranks, one block-wide scan over the bucket counts);
+//   3. each wavefront walks its share of the grouped records with lane = feature (64 / PW records per
+//      instruction), recomputes each pair's contribution w * (g_mean / K + [argmax == slot] * g_max) from the rows
+//      kept in LDS, sums it in a register while the target stays the same, and issues ONE row update per run of
+//      equal targets.
+// For 32 rows with K = 40 (64) that is 3.7 (4.1) times fewer updates (sampled on learned 4-D coordinates), and the
+// result is the same sum in another order.
+#ifndef TILE_ABL
+#define TILE_ABL 0
+#endif
 #ifndef GT
-#define GT 8             // sorted rows per wavefront (16: fewer row updates, but the longer serial walk of step 3 and
-#endif                   // half the wavefronts per CU cost more than they save: 1.15 against 0.84 ms at N=300k, K=40, P=32)
+#define GT 8             // sorted rows per wavefront
+#endif
+#ifndef GT_WAVES
+#define GT_WAVES 4       // wavefronts per block: the block's tile is GT_WAVES * GT rows
+#endif
 #ifndef GT_BUCKETS
-#define GT_BUCKETS 512
+#define GT_BUCKETS 1024  // buckets of the counting sort (two targets that share a bucket split each other's runs)
 #endif
 
 template <int PW>
-__global__ __launch_bounds__(64) void k_gravnet_bwd_tile(const int *__restrict__ nbr, const uint32_t *__restrict__ order,
-                                                         const float *__restrict__ dsq, const float *__restrict__ feat,
-                                                         int ldf, const int *__restrict__ argmax,
-                                                         const float *__restrict__ gmean,
-                                                         const float *__restrict__ gmax, int ldg,
-                                                         float *__restrict__ gfeat, int ldgf,
-                                                         float *__restrict__ gdsq, int64_t n, int K, int P,
-                                                         int *__restrict__ status)
+__global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
+    const int *__restrict__ nbr, const uint32_t *__restrict__ order, const float *__restrict__ dsq,
+    const float *__restrict__ feat, int ldf, const int *__restrict__ argmax, const float *__restrict__ gmean,
+    const float *__restrict__ gmax, int ldg, float *__restrict__ gfeat, int ldgf, float *__restrict__ gdsq, int64_t n,
+    int K, int P, int *__restrict__ status)
 {
     constexpr int QPW = 64 / PW;               // rows per pass of step 1b, records per instruction of step 3
-    static_assert(GT % QPW == 0 && GT <= 64, "tile rows");
+    constexpr int GTB = GT_WAVES * GT;         // rows of the block's tile
+    constexpr int NSEG3 = GT_WAVES * QPW;      // lane groups that share the walk of step 3
+    constexpr int BPT = GT_BUCKETS / (GT_WAVES * 64);   // buckets per thread in the scan
+    static_assert(GT % QPW == 0 && GTB <= 256 && GT_BUCKETS % (GT_WAVES * 64) == 0, "tile shape");
     extern __shared__ __align__(16) unsigned char s_raw[];
     const int lane = fgc_lane();
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int sub = lane / PW, pl = lane % PW;
-    // LDS: upstream rows [GT][PW] x 3, bucket counts, then the records: first as three arrays (target position,
-    // weight, target's original index) indexed [row][slot], later - over the same bytes - as 16-byte grouped records
-    float *rows_cm = (float *)s_raw;
-    float *rows_gx = rows_cm + GT * PW;
-    int *rows_am = (int *)(rows_gx + GT * PW);
-    int *hist = rows_am + GT * PW;
-    unsigned char *rec0 = (unsigned char *)(hist + GT_BUCKETS);
+    // LDS: upstream rows [GTB][PW] (two floats and the arg-max slot as a byte), bucket counts, the wavefronts' record
+    // totals, then the records: first as three arrays (target position, weight, target's original index) indexed
+    // [row][slot], later - over the same bytes - as three arrays of the grouped records (target's original index,
+    // weight, row and slot), padded for the walk of step 3
+    const int E = GTB * K, EP = E + 4 * NSEG3;
+    float2 *rows_cg = (float2 *)s_raw;
+    int *hist = (int *)(rows_cg + GTB * PW);
+    int *wsum = hist + GT_BUCKETS;
+    unsigned char *rec0 = (unsigned char *)(wsum + 4 * ((GT_WAVES + 3) / 4));
     int *em = (int *)rec0;
-    float *ew = (float *)(em + GT * K);
-    int *eo = (int *)(ew + GT * K);
-    uint4 *srec = (uint4 *)rec0;
-    const int64_t r0 = (int64_t)blockIdx.x * GT;
+    float *ew = (float *)(em + E);
+    int *eo = (int *)(ew + E);
+    int *st = (int *)rec0;
+    float *sw = (float *)(st + EP);
+    int *sz = (int *)(sw + EP);
+    unsigned char *rows_am = (unsigned char *)(sz + EP);
+    const int tw0 = wv * GT;                                      // the wavefront's first row inside the tile
+    const int64_t r0 = (int64_t)blockIdx.x * GTB + tw0;           // ... and in the sorted order
     const float invK = 1.0f / (float)K;
     const unsigned ldf4 = 4u * (unsigned)ldf;
     bool bad = false;
-    for (int t = lane; t < GT_BUCKETS; t += 64) hist[t] = 0;
+    for (int t = threadIdx.x; t < GT_BUCKETS; t += GT_WAVES * 64) hist[t] = 0;
 
-    // ---- 1a. everything the tile needs except the feature gathers, all loads independent of each other:
-    //      lane t keeps row t's original index; per row (lane = slot) the neighbour positions, their weights and
-    //      original indices go to LDS; per QPW rows (lane = feature) the upstream gradients and arg-max slots ----
+    // ---- 1a. everything the wavefront's rows need except the feature gathers, all loads independent of each
+    //      other: lane t keeps row t's original index; per row (lane = slot) the neighbour positions, their weights
+    //      and original indices go to LDS (the positions also stay in registers for step 2); per QPW rows (lane =
+    //      feature) the upstream gradients and arg-max slots ----
     const unsigned my_qo = (lane < GT && r0 + lane < n) ? order[r0 + lane] : 0u;
-#pragma unroll 4
+    int rm[GT];
+#pragma unroll
     for (int t = 0; t < GT; t++) {
         const bool qv = r0 + t < n;
         const int64_t qo = (int64_t)(unsigned)fgc_readlane_i((int)my_qo, t);
@@ -901,41 +918,42 @@ __global__ __launch_bounds__(64) void k_gravnet_bwd_tile(const int *__restrict__
             if (m >= n) { bad = true; m = -1; }
             if (m >= 0) o = (int)order[m];
         }
-        if (lane < K) { em[t * K + lane] = m; ew[t * K + lane] = w; eo[t * K + lane] = o; }
+        rm[t] = m;
+        if (lane < K) { em[(tw0 + t) * K + lane] = m; ew[(tw0 + t) * K + lane] = w; eo[(tw0 + t) * K + lane] = o; }
     }
     for (int t0 = 0; t0 < GT; t0 += QPW) {
         const int t = t0 + sub;
         const bool qv = r0 + t < n;
         const int64_t qo = (int64_t)(unsigned)__shfl((int)my_qo, t, 64);
         float cm = 0.f, gx = 0.f;
-        int am = -1;
+        int am = 255;
         if (qv && pl < P) {
             cm = gmean[qo * ldg + pl] * invK;
             gx = gmax[qo * ldg + pl];
-            am = argmax[qo * P + pl];
+            am = argmax[qo * P + pl] & 255;          // slots are < 64; -1 (no neighbour) becomes 255
         }
-        rows_cm[t * PW + pl] = cm;
-        rows_gx[t * PW + pl] = gx;
-        rows_am[t * PW + pl] = am;
+        rows_cg[(tw0 + t) * PW + pl] = make_float2(cm, gx);
+        rows_am[(tw0 + t) * PW + pl] = (unsigned char)am;
     }
 
     // ---- 1b. dot products for grad_distsq: lane = feature, QPW rows at a time, eight slots per step; the feature
     //      gathers of the next step are requested before the current one is reduced ----
     const int n_grp = (K + 7) >> 3;
     for (int t0 = 0; t0 < GT; t0 += QPW) {
-        const int t = t0 + sub;
+        const int t = t0 + sub, tb = tw0 + t;
         const bool qv = r0 + t < n;
         const int64_t qo = (int64_t)(unsigned)__shfl((int)my_qo, t, 64);
-        const float cm = rows_cm[t * PW + pl], gx = rows_gx[t * PW + pl];
-        const int am = rows_am[t * PW + pl];
+        const float2 cg = rows_cg[tb * PW + pl];
+        const float cm = cg.x, gx = cg.y;
+        const int am = rows_am[tb * PW + pl];
         auto gather = [&](int g, float (&f)[8]) {
 #pragma unroll
             for (int u = 0; u < 8; u++) {
                 const int k = g * 8 + u;
                 f[u] = 0.f;
                 if (k < K && pl < P) {
-                    const int mu = em[t * K + k];
-                    if (mu >= 0) f[u] = *(const float *)((const char *)feat + (__umul24((unsigned)eo[t * K + k], ldf4) + 4u * (unsigned)pl));
+                    const int mu = em[tb * K + k];
+                    if (mu >= 0) f[u] = *(const float *)((const char *)feat + (__umul24((unsigned)eo[tb * K + k], ldf4) + 4u * (unsigned)pl));
                 }
             }
         };
@@ -948,73 +966,97 @@ __global__ __launch_bounds__(64) void k_gravnet_bwd_tile(const int *__restrict__
             for (int u = 0; u < 8; u++) vals[u] = fcur[u] * (cm + (am == g * 8 + u ? gx : 0.f));
             const float tot = fgc_group_reduce8<PW>(vals, lane);
             const int k = g * 8 + pl * 8 / PW;          // the slot whose total the lane holds
-            if (qv && (pl % (PW / 8)) == 0 && k < K) gdsq[qo * K + k] = -10.f * ew[t * K + k] * tot;
+            if (qv && (pl % (PW / 8)) == 0 && k < K) gdsq[qo * K + k] = -10.f * ew[tb * K + k] * tot;
 #pragma unroll
             for (int u = 0; u < 8; u++) fcur[u] = fnext[u];
         }
     }
+#if TILE_ABL == 1
+    return;
+#endif
 
-    // ---- 2. group the records by target: counting sort on the low bits of the target's sorted position ----
-    int rm[GT], ro[GT], rp[GT];
+    // ---- 2. group the block's records by target: counting sort on the low bits of the target's sorted position ----
+    __syncthreads();                                  // the bucket counts are zero
+    int ro[GT], rp[GT];
     float rw[GT];
 #pragma unroll
-    for (int t = 0; t < GT; t++) {                    // lane = slot of row t
-        rm[t] = -1; ro[t] = 0; rp[t] = 0; rw[t] = 0.f;
-        if (lane < K) { rm[t] = em[t * K + lane]; rw[t] = ew[t * K + lane]; ro[t] = eo[t * K + lane]; }
+    for (int t = 0; t < GT; t++) {                    // lane = slot of the wavefront's row t
+        ro[t] = 0; rp[t] = 0; rw[t] = 0.f;
+        if (lane < K) { rw[t] = ew[(tw0 + t) * K + lane]; ro[t] = eo[(tw0 + t) * K + lane]; }
         if (rm[t] >= 0) rp[t] = atomicAdd(&hist[rm[t] & (GT_BUCKETS - 1)], 1);     // rank inside the bucket
     }
-    asm volatile("" ::: "memory");     // the records are read before anything is written over them (other types below)
-    // exclusive scan of the bucket counts: consecutive buckets per lane, then across the lanes
-    int cntv[GT_BUCKETS / 64], run = 0;
+    __syncthreads();                                  // all ranks taken, every record of the block is in registers
+    // exclusive scan of the bucket counts: consecutive buckets per thread, across the lanes, across the wavefronts
+    int cntv[BPT], run = 0;
+    const int b0 = (int)threadIdx.x * BPT;
 #pragma unroll
-    for (int b = 0; b < GT_BUCKETS / 64; b++) { cntv[b] = hist[lane * (GT_BUCKETS / 64) + b]; run += cntv[b]; }
+    for (int b = 0; b < BPT; b++) { cntv[b] = hist[b0 + b]; run += cntv[b]; }
     int incl = run;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
         const int up = __shfl_up(incl, o, 64);
         if (lane >= o) incl += up;
     }
-    const int n_rec = __shfl(incl, 63, 64);
-    int base = incl - run;
+    if (lane == 63) wsum[wv] = incl;
+    __syncthreads();
+    int woff = 0, n_rec = 0;
 #pragma unroll
-    for (int b = 0; b < GT_BUCKETS / 64; b++) { hist[lane * (GT_BUCKETS / 64) + b] = base; base += cntv[b]; }
-    // every record is in registers by now: the grouped records may overwrite the three arrays
+    for (int v = 0; v < GT_WAVES; v++) { const int c = wsum[v]; woff += v < wv ? c : 0; n_rec += c; }
+    int base = woff + incl - run;
+#pragma unroll
+    for (int b = 0; b < BPT; b++) { hist[b0 + b] = base; base += cntv[b]; }
+    __syncthreads();                                  // bucket offsets complete
+    // the grouped records overwrite the three arrays (every record is in registers since the second barrier); the
+    // walk below takes whole groups of four records per lane group: the rest is padded with records of weight 0
+    // for target -1
+    const int per = ((n_rec + NSEG3 - 1) / NSEG3 + 3) & ~3;
 #pragma unroll
     for (int t = 0; t < GT; t++) {
         if (rm[t] >= 0) {
             const int dst = hist[rm[t] & (GT_BUCKETS - 1)] + rp[t];
-            srec[dst] = make_uint4((unsigned)ro[t], __float_as_uint(rw[t]), (unsigned)((t << 8) | lane), (unsigned)rm[t]);
+            st[dst] = ro[t]; sw[dst] = rw[t]; sz[dst] = ((tw0 + t) << 8) | lane;
         }
     }
+    for (int j = n_rec + (int)threadIdx.x; j < NSEG3 * per; j += GT_WAVES * 64) { st[j] = -1; sw[j] = 0.f; sz[j] = 0; }
+    __syncthreads();
+#if TILE_ABL == 3
+    return;
+#endif
 
-    // ---- 3. one row update per run of equal targets; lane = feature, QPW records per instruction ----
-    const int per = (n_rec + QPW - 1) / QPW;
-    const int j_beg = sub * per, j_end = min(n_rec, j_beg + per);
+    // ---- 3. one row update per run of equal targets; lane = feature, QPW records per instruction, the grouped
+    //      records split evenly over the block's lane groups; the next four records are requested before the
+    //      current four are used ----
+    const int j_beg = (wv * QPW + sub) * per;
     int cur = -1;
     float acc = 0.f;
+    int4 t4 = *(const int4 *)&st[j_beg], z4 = *(const int4 *)&sz[j_beg];
+    float4 w4 = *(const float4 *)&sw[j_beg];
     for (int j = j_beg; j < j_beg + per; j += 4) {
-        uint4 rc[4];
-        float cmv[4], gxv[4];
+        const int tg[4] = {t4.x, t4.y, t4.z, t4.w}, zz[4] = {z4.x, z4.y, z4.z, z4.w};
+        const float ww[4] = {w4.x, w4.y, w4.z, w4.w};
+        if (j + 4 < j_beg + per) {
+            t4 = *(const int4 *)&st[j + 4]; z4 = *(const int4 *)&sz[j + 4]; w4 = *(const float4 *)&sw[j + 4];
+        }
+        float2 cgv[4];
         int amv[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            rc[u] = (j + u < j_end) ? srec[j + u] : make_uint4(0xffffffffu, 0u, 0u, 0u);
-            const int t = (int)(rc[u].z >> 8) & (GT - 1);
-            cmv[u] = rows_cm[t * PW + pl];
-            gxv[u] = rows_gx[t * PW + pl];
+            const int t = (zz[u] >> 8) & (GTB - 1);
+            cgv[u] = rows_cg[t * PW + pl];
             amv[u] = rows_am[t * PW + pl];
         }
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            const int tgt = (int)rc[u].x;
-            if (j + u < j_end) {
-                if (tgt != cur) {
-                    if (cur >= 0 && cur < n && pl < P) atomicAdd(&gfeat[(int64_t)cur * ldgf + pl], acc);
-                    cur = tgt;
-                    acc = 0.f;
-                }
-                acc += __uint_as_float(rc[u].y) * (cmv[u] + (amv[u] == (int)(rc[u].z & 255u) ? gxv[u] : 0.f));
+            if (tg[u] != cur) {
+#if TILE_ABL == 2
+                if (cur >= 0 && cur < n && pl < P && acc == 1.2345f) gfeat[(int64_t)cur * ldgf + pl] = acc;
+#else
+                if (cur >= 0 && cur < n && pl < P) atomicAdd(&gfeat[(int64_t)cur * ldgf + pl], acc);
+#endif
+                cur = tg[u];
+                acc = 0.f;
             }
+            acc += ww[u] * (cgv[u].x + (amv[u] == (zz[u] & 255) ? cgv[u].y : 0.f));
         }
     }
     if (cur >= 0 && cur < n && pl < P) atomicAdd(&gfeat[(int64_t)cur * ldgf + pl], acc);
@@ -1023,7 +1065,8 @@ __global__ __launch_bounds__(64) void k_gravnet_bwd_tile(const int *__restrict__
 
 static size_t gravnet_tile_lds(int pw, int K)
 {
-    return (size_t)GT * pw * 12 + (size_t)GT_BUCKETS * 4 + (size_t)GT * K * 16;
+    const size_t rows = (size_t)GT_WAVES * GT, nseg3 = (size_t)GT_WAVES * (64 / pw);
+    return rows * pw * 9 + (size_t)GT_BUCKETS * 4 + 16 * ((GT_WAVES + 3) / 4) + 12 * (rows * K + 4 * nseg3);
 }
 
 static int pick_pw(int P)
@@ -1121,10 +1164,20 @@ extern "C" int fgc_gravnet_aggregate_bwd_sorted_f32(const int32_t *d_nbr_sorted,
         return FGC_EINVAL;
     hipStream_t s = (hipStream_t)stream;
     const int pw = pick_pw(P);
-    const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GT);
+    const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GT_WAVES * GT);
     const size_t lds = gravnet_tile_lds(pw, K);
+    // more than 64 KB of dynamic LDS per block (P > 32 with K = 64) has to be granted per kernel, once
 #define FGC_L(PWW)                                                                                              \
-    hipLaunchKernelGGL((k_gravnet_bwd_tile<PWW>), dim3(blocks), dim3(64), lds, s, d_nbr_sorted,                \
+    if (lds > 65536) {                                                                                          \
+        static std::atomic<size_t> granted{0};                                                                  \
+        if (granted.load() < lds) {                                                                             \
+            if (hipFuncSetAttribute((const void *)k_gravnet_bwd_tile<PWW>,                                      \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)        \
+                return FGC_EUNSUPPORTED;                                                                        \
+            granted.store(lds);                                                                                 \
+        }                                                                                                       \
+    }                                                                                                           \
+    hipLaunchKernelGGL((k_gravnet_bwd_tile<PWW>), dim3(blocks), dim3(GT_WAVES * 64), lds, s, d_nbr_sorted,      \
                        (const uint32_t *)d_order, d_distsq, d_feat, (int)ld_feat, d_argmax, d_grad_fmean,      \
                        d_grad_fmax, (int)ld_grad, d_grad_feat, (int)ld_grad_feat, d_grad_distsq, n_vert, (int)K, \
                        (int)P, d_status)
