@@ -881,13 +881,13 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
     // totals, then the records: first as three arrays (target position, weight, target's original index) indexed
     // [row][slot], later - over the same bytes - as three arrays of the grouped records (target's original index,
     // weight, row and slot), padded for the walk of step 3
-    const int E = GTB * K, EP = E + 4 * NSEG3;
+    const int KP = (K + 7) & ~7;               // slots per row in LDS, padded to whole groups of eight
+    const int E = GTB * KP, EP = E + 4 * NSEG3;
     float2 *rows_cg = (float2 *)s_raw;
     int *hist = (int *)(rows_cg + GTB * PW);
     int *wsum = hist + GT_BUCKETS;
     unsigned char *rec0 = (unsigned char *)(wsum + 4 * ((GT_WAVES + 3) / 4));
-    int *em = (int *)rec0;
-    float *ew = (float *)(em + E);
+    float *ew = (float *)rec0;
     int *eo = (int *)(ew + E);
     int *st = (int *)rec0;
     float *sw = (float *)(st + EP);
@@ -910,7 +910,7 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
     for (int t = 0; t < GT; t++) {
         const bool qv = r0 + t < n;
         const int64_t qo = (int64_t)(unsigned)fgc_readlane_i((int)my_qo, t);
-        int m = -1, o = 0;
+        int m = -1, o = -1;                      // no neighbour: original index -1
         float w = 0.f;
         if (qv && lane < K) {
             m = nbr[(r0 + t) * K + lane];
@@ -919,7 +919,7 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
             if (m >= 0) o = (int)order[m];
         }
         rm[t] = m;
-        if (lane < K) { em[(tw0 + t) * K + lane] = m; ew[(tw0 + t) * K + lane] = w; eo[(tw0 + t) * K + lane] = o; }
+        if (lane < KP) { ew[(tw0 + t) * KP + lane] = w; eo[(tw0 + t) * KP + lane] = o; }
     }
     for (int t0 = 0; t0 < GT; t0 += QPW) {
         const int t = t0 + sub;
@@ -939,6 +939,7 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
     // ---- 1b. dot products for grad_distsq: lane = feature, QPW rows at a time, eight slots per step; the feature
     //      gathers of the next step are requested before the current one is reduced ----
     const int n_grp = (K + 7) >> 3;
+#if TILE_ABL != 4
     for (int t0 = 0; t0 < GT; t0 += QPW) {
         const int t = t0 + sub, tb = tw0 + t;
         const bool qv = r0 + t < n;
@@ -947,14 +948,17 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
         const float cm = cg.x, gx = cg.y;
         const int am = rows_am[tb * PW + pl];
         auto gather = [&](int g, float (&f)[8]) {
+            // the eight original indices of the group with two 16-byte LDS reads
+            const int4 oa = *(const int4 *)&eo[tb * KP + g * 8], ob = *(const int4 *)&eo[tb * KP + g * 8 + 4];
+            const int oo[8] = {oa.x, oa.y, oa.z, oa.w, ob.x, ob.y, ob.z, ob.w};
 #pragma unroll
             for (int u = 0; u < 8; u++) {
-                const int k = g * 8 + u;
                 f[u] = 0.f;
-                if (k < K && pl < P) {
-                    const int mu = em[tb * K + k];
-                    if (mu >= 0) f[u] = *(const float *)((const char *)feat + (__umul24((unsigned)eo[tb * K + k], ldf4) + 4u * (unsigned)pl));
-                }
+#if TILE_ABL == 5
+                if (oo[u] >= 0 && pl < P) f[u] = __uint_as_float(__umul24((unsigned)oo[u], ldf4) + 4u * (unsigned)pl);
+#else
+                if (oo[u] >= 0 && pl < P) f[u] = *(const float *)((const char *)feat + (__umul24((unsigned)oo[u], ldf4) + 4u * (unsigned)pl));
+#endif
             }
         };
         float fcur[8], fnext[8];
@@ -966,11 +970,12 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
             for (int u = 0; u < 8; u++) vals[u] = fcur[u] * (cm + (am == g * 8 + u ? gx : 0.f));
             const float tot = fgc_group_reduce8<PW>(vals, lane);
             const int k = g * 8 + pl * 8 / PW;          // the slot whose total the lane holds
-            if (qv && (pl % (PW / 8)) == 0 && k < K) gdsq[qo * K + k] = -10.f * ew[tb * K + k] * tot;
+            if (qv && (pl % (PW / 8)) == 0 && k < K) gdsq[qo * K + k] = -10.f * ew[tb * KP + k] * tot;
 #pragma unroll
             for (int u = 0; u < 8; u++) fcur[u] = fnext[u];
         }
     }
+#endif
 #if TILE_ABL == 1
     return;
 #endif
@@ -982,7 +987,7 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
 #pragma unroll
     for (int t = 0; t < GT; t++) {                    // lane = slot of the wavefront's row t
         ro[t] = 0; rp[t] = 0; rw[t] = 0.f;
-        if (lane < K) { rw[t] = ew[(tw0 + t) * K + lane]; ro[t] = eo[(tw0 + t) * K + lane]; }
+        if (lane < K) { rw[t] = ew[(tw0 + t) * KP + lane]; ro[t] = eo[(tw0 + t) * KP + lane]; }
         if (rm[t] >= 0) rp[t] = atomicAdd(&hist[rm[t] & (GT_BUCKETS - 1)], 1);     // rank inside the bucket
     }
     __syncthreads();                                  // all ranks taken, every record of the block is in registers
@@ -1014,7 +1019,7 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
     for (int t = 0; t < GT; t++) {
         if (rm[t] >= 0) {
             const int dst = hist[rm[t] & (GT_BUCKETS - 1)] + rp[t];
-            st[dst] = ro[t]; sw[dst] = rw[t]; sz[dst] = ((tw0 + t) << 8) | lane;
+            st[dst] = ro[t]; sw[dst] = rw[t]; sz[dst] = (((tw0 + t) * PW) << 8) | lane;
         }
     }
     for (int j = n_rec + (int)threadIdx.x; j < NSEG3 * per; j += GT_WAVES * 64) { st[j] = -1; sw[j] = 0.f; sz[j] = 0; }
@@ -1027,46 +1032,61 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
     //      records split evenly over the block's lane groups; the next four records are requested before the
     //      current four are used ----
     const int j_beg = (wv * QPW + sub) * per;
+    const unsigned n_l = pl < P ? (unsigned)n : 0u;            // lanes without a feature never pass the bound check
+    const unsigned ldgf4 = 4u * (unsigned)ldgf;
+    char *const gbase = (char *)gfeat + 4 * pl;
     int cur = -1;
     float acc = 0.f;
-    int4 t4 = *(const int4 *)&st[j_beg], z4 = *(const int4 *)&sz[j_beg];
-    float4 w4 = *(const float4 *)&sw[j_beg];
-    for (int j = j_beg; j < j_beg + per; j += 4) {
+    auto flush = [&]() {
+#if TILE_ABL == 2
+        if ((unsigned)cur < n_l && acc == 1.2345f) *(float *)(gbase + __umul24((unsigned)cur, ldgf4)) = acc;
+#else
+        if ((unsigned)cur < n_l) atomicAdd((float *)(gbase + __umul24((unsigned)cur, ldgf4)), acc);
+#endif
+    };
+    auto load4 = [&](int j, int4 &t4, int4 &z4, float4 &w4) {
+        t4 = *(const int4 *)&st[j]; z4 = *(const int4 *)&sz[j]; w4 = *(const float4 *)&sw[j];
+    };
+    auto use4 = [&](const int4 &t4, const int4 &z4, const float4 &w4) {
         const int tg[4] = {t4.x, t4.y, t4.z, t4.w}, zz[4] = {z4.x, z4.y, z4.z, z4.w};
         const float ww[4] = {w4.x, w4.y, w4.z, w4.w};
-        if (j + 4 < j_beg + per) {
-            t4 = *(const int4 *)&st[j + 4]; z4 = *(const int4 *)&sz[j + 4]; w4 = *(const float4 *)&sw[j + 4];
-        }
         float2 cgv[4];
         int amv[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            const int t = (zz[u] >> 8) & (GTB - 1);
-            cgv[u] = rows_cg[t * PW + pl];
-            amv[u] = rows_am[t * PW + pl];
+            const int ri = (zz[u] >> 8) + pl;            // the record names its row as row * PW
+            cgv[u] = rows_cg[ri];
+            amv[u] = rows_am[ri];
         }
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             if (tg[u] != cur) {
-#if TILE_ABL == 2
-                if (cur >= 0 && cur < n && pl < P && acc == 1.2345f) gfeat[(int64_t)cur * ldgf + pl] = acc;
-#else
-                if (cur >= 0 && cur < n && pl < P) atomicAdd(&gfeat[(int64_t)cur * ldgf + pl], acc);
-#endif
+                flush();
                 cur = tg[u];
                 acc = 0.f;
             }
             acc += ww[u] * (cgv[u].x + (amv[u] == (zz[u] & 255) ? cgv[u].y : 0.f));
         }
+    };
+    int4 ta, za, tb4, zb;
+    float4 wa, wb;
+    load4(j_beg, ta, za, wa);                       // per = 0: reads inside the arrays, uses nothing
+    int i = 0;
+    for (; i + 8 <= per; i += 8) {                  // two groups of four per pass: no register copies
+        load4(j_beg + i + 4, tb4, zb, wb);
+        use4(ta, za, wa);
+        if (i + 8 < per) load4(j_beg + i + 8, ta, za, wa);
+        use4(tb4, zb, wb);
     }
-    if (cur >= 0 && cur < n && pl < P) atomicAdd(&gfeat[(int64_t)cur * ldgf + pl], acc);
+    if (i < per) use4(ta, za, wa);
+    flush();
     if (bad && status) atomicOr(&status[0], FGC_ST_BAD_INDEX);
 }
 
 static size_t gravnet_tile_lds(int pw, int K)
 {
     const size_t rows = (size_t)GT_WAVES * GT, nseg3 = (size_t)GT_WAVES * (64 / pw);
-    return rows * pw * 9 + (size_t)GT_BUCKETS * 4 + 16 * ((GT_WAVES + 3) / 4) + 12 * (rows * K + 4 * nseg3);
+    return rows * pw * 9 + (size_t)GT_BUCKETS * 4 + 16 * ((GT_WAVES + 3) / 4) + 12 * (rows * ((K + 7) & ~7) + 4 * nseg3);
 }
 
 static int pick_pw(int P)
@@ -1155,8 +1175,9 @@ extern "C" int fgc_gravnet_aggregate_bwd_sorted_f32(const int32_t *d_nbr_sorted,
 {
     if (n_vert < 0 || K < 1 || P < 1 || ld_feat < P || ld_grad < P || ld_grad_feat < P) return FGC_EINVAL;
     if (K > 64 || P > 64 || P <= 8 || n_vert >= (1ll << 31) - 1) return FGC_EUNSUPPORTED;
-    // 32-bit byte offsets of the feature rows, formed with a 24-bit multiply
-    if (n_vert >= (1 << 24) || ld_feat >= (1 << 22) || (uint64_t)n_vert * (uint64_t)ld_feat * 4ull >= 0xffffffffull)
+    // 32-bit byte offsets of the feature and gradient rows, formed with a 24-bit multiply
+    if (n_vert >= (1 << 24) || ld_feat >= (1 << 22) || (uint64_t)n_vert * (uint64_t)ld_feat * 4ull >= 0xffffffffull ||
+        ld_grad_feat >= (1 << 22) || (uint64_t)n_vert * (uint64_t)ld_grad_feat * 4ull >= 0xffffffffull)
         return FGC_EUNSUPPORTED;
     if (n_vert == 0) return FGC_OK;
     if (!d_nbr_sorted || !d_order || !d_distsq || !d_feat || !d_argmax || !d_grad_fmean || !d_grad_fmax ||
