@@ -14,7 +14,7 @@ collect_stats = False
 # returned are the same either way; only the run time differs.
 auto_grid = True
 
-# GravNetOp's backward: combine the feature gradients of 8 rows that are consecutive in the search's sorted order
+# GravNetOp's backward: combine the feature gradients of 32 rows that are consecutive in the search's sorted order
 # on chip before they are added to memory (K <= 64, 8 < P <= 64).  False: one atomic row update per (point, slot)
 # pair, the kernel the stand-alone gravnet_aggregate op uses.  Same gradients up to float summation order.
 tile_aggregation_backward = True

@@ -837,20 +837,20 @@ __global__ __launch_bounds__(256) void k_gravnet_bwd(const int64_t *__restrict__
 // k_gravnet_bwd issues one atomic 128-byte row update per (point, slot) pair and is bound by the rate of those
 // updates.  Rows that are consecutive in the sorted order share most of their neighbours, so a block of GT_WAVES
 // wavefronts here takes GT_WAVES * GT consecutive sorted rows and
-//   1. each wavefront loads what its GT rows need into LDS (per pair a record: target, weight; per row the upstream
-//      gradients and arg-max slots), then, per row pair with lane = feature, gathers the neighbours' feature rows
-//      and forms the dot products for grad_distsq as k_gravnet_bwd does - but does not touch grad_feat;
+//   1. each wavefront loads what its GT rows need into LDS (per pair the weight and the target's original index -
+//      the target's sorted position stays in a register; per row the upstream gradients and arg-max slots), then,
+//      per row pair with lane = feature, gathers the neighbours' feature rows and forms the dot products for
+//      grad_distsq as k_gravnet_bwd does - but does not touch grad_feat;
 //   2. the block groups all its records by target with a counting sort on the low bits of the target's sorted
 //      position (lane = record; LDS integer atomics for the ranks, one block-wide scan over the bucket counts);
 //   3. each wavefront walks its share of the grouped records with lane = feature (64 / PW records per
-//      instruction), recomputes each pair's contribution w * (g_mean / K + [argmax == slot] * g_max) from the rows
-//      kept in LDS, sums it in a register while the target stays the same, and issues ONE row update per run of
-//      equal targets.
-// For 32 rows with K = 40 (64) that is 3.7 (4.1) times fewer updates (sampled on learned 4-D coordinates), and the
-// result is the same sum in another order.
-#ifndef TILE_ABL
-#define TILE_ABL 0
-#endif
+//      instruction, four records per 16-byte LDS read, the next four requested before the current four are used),
+//      recomputes each pair's contribution w * (g_mean / K + [argmax == slot] * g_max) from the rows kept in LDS,
+//      sums it in a register while the target stays the same, and issues ONE row update per run of equal targets.
+// For 32 rows with K = 40 (64) that is 3.5 (3.9) times fewer updates (sampled on learned 4-D coordinates, 1024
+// buckets), and the result is the same sum in another order.  What the block needs in LDS decides how many
+// wavefronts a CU holds, and the kernel's time follows that number: 9 bytes per (row, feature), 4 KB of bucket
+// counts and 12 bytes per pair - 38 KB at K = 64, P = 32 (four blocks per CU), 29 KB at K = 40 (five).
 #ifndef GT
 #define GT 8             // sorted rows per wavefront
 #endif
@@ -877,10 +877,10 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
     const int lane = fgc_lane();
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int sub = lane / PW, pl = lane % PW;
-    // LDS: upstream rows [GTB][PW] (two floats and the arg-max slot as a byte), bucket counts, the wavefronts' record
-    // totals, then the records: first as three arrays (target position, weight, target's original index) indexed
-    // [row][slot], later - over the same bytes - as three arrays of the grouped records (target's original index,
-    // weight, row and slot), padded for the walk of step 3
+    // LDS: upstream rows [GTB][PW] (g_mean / K without and with g_max added, and the arg-max slot as a byte), bucket
+    // counts, the wavefronts' record totals, then the pairs: first as two arrays (weight, target's original index)
+    // indexed [row][slot], later - over the same bytes - as three arrays of the grouped records (target's original
+    // index, weight, row and slot), padded for the walk of step 3
     const int KP = (K + 7) & ~7;               // slots per row in LDS, padded to whole groups of eight
     const int E = GTB * KP, EP = E + 4 * NSEG3;
     float2 *rows_cg = (float2 *)s_raw;
@@ -932,20 +932,19 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
             gx = gmax[qo * ldg + pl];
             am = argmax[qo * P + pl] & 255;          // slots are < 64; -1 (no neighbour) becomes 255
         }
-        rows_cg[(tw0 + t) * PW + pl] = make_float2(cm, gx);
+        rows_cg[(tw0 + t) * PW + pl] = make_float2(cm, cm + gx);      // without and with the arg-max share
         rows_am[(tw0 + t) * PW + pl] = (unsigned char)am;
     }
 
     // ---- 1b. dot products for grad_distsq: lane = feature, QPW rows at a time, eight slots per step; the feature
     //      gathers of the next step are requested before the current one is reduced ----
     const int n_grp = (K + 7) >> 3;
-#if TILE_ABL != 4
     for (int t0 = 0; t0 < GT; t0 += QPW) {
         const int t = t0 + sub, tb = tw0 + t;
         const bool qv = r0 + t < n;
         const int64_t qo = (int64_t)(unsigned)__shfl((int)my_qo, t, 64);
         const float2 cg = rows_cg[tb * PW + pl];
-        const float cm = cg.x, gx = cg.y;
+        const float cm = cg.x, cmgx = cg.y;
         const int am = rows_am[tb * PW + pl];
         auto gather = [&](int g, float (&f)[8]) {
             // the eight original indices of the group with two 16-byte LDS reads
@@ -954,11 +953,7 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
 #pragma unroll
             for (int u = 0; u < 8; u++) {
                 f[u] = 0.f;
-#if TILE_ABL == 5
-                if (oo[u] >= 0 && pl < P) f[u] = __uint_as_float(__umul24((unsigned)oo[u], ldf4) + 4u * (unsigned)pl);
-#else
                 if (oo[u] >= 0 && pl < P) f[u] = *(const float *)((const char *)feat + (__umul24((unsigned)oo[u], ldf4) + 4u * (unsigned)pl));
-#endif
             }
         };
         float fcur[8], fnext[8];
@@ -967,7 +962,7 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
             if (g + 1 < n_grp) gather(g + 1, fnext);
             float vals[8];
 #pragma unroll
-            for (int u = 0; u < 8; u++) vals[u] = fcur[u] * (cm + (am == g * 8 + u ? gx : 0.f));
+            for (int u = 0; u < 8; u++) vals[u] = fcur[u] * (am == g * 8 + u ? cmgx : cm);
             const float tot = fgc_group_reduce8<PW>(vals, lane);
             const int k = g * 8 + pl * 8 / PW;          // the slot whose total the lane holds
             if (qv && (pl % (PW / 8)) == 0 && k < K) gdsq[qo * K + k] = -10.f * ew[tb * KP + k] * tot;
@@ -975,10 +970,6 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
             for (int u = 0; u < 8; u++) fcur[u] = fnext[u];
         }
     }
-#endif
-#if TILE_ABL == 1
-    return;
-#endif
 
     // ---- 2. group the block's records by target: counting sort on the low bits of the target's sorted position ----
     __syncthreads();                                  // the bucket counts are zero
@@ -1024,9 +1015,6 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
     }
     for (int j = n_rec + (int)threadIdx.x; j < NSEG3 * per; j += GT_WAVES * 64) { st[j] = -1; sw[j] = 0.f; sz[j] = 0; }
     __syncthreads();
-#if TILE_ABL == 3
-    return;
-#endif
 
     // ---- 3. one row update per run of equal targets; lane = feature, QPW records per instruction, the grouped
     //      records split evenly over the block's lane groups; the next four records are requested before the
@@ -1038,11 +1026,7 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
     int cur = -1;
     float acc = 0.f;
     auto flush = [&]() {
-#if TILE_ABL == 2
-        if ((unsigned)cur < n_l && acc == 1.2345f) *(float *)(gbase + __umul24((unsigned)cur, ldgf4)) = acc;
-#else
         if ((unsigned)cur < n_l) atomicAdd((float *)(gbase + __umul24((unsigned)cur, ldgf4)), acc);
-#endif
     };
     auto load4 = [&](int j, int4 &t4, int4 &z4, float4 &w4) {
         t4 = *(const int4 *)&st[j]; z4 = *(const int4 *)&sz[j]; w4 = *(const float4 *)&sw[j];
@@ -1065,7 +1049,7 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
                 cur = tg[u];
                 acc = 0.f;
             }
-            acc += ww[u] * (cgv[u].x + (amv[u] == (zz[u] & 255) ? cgv[u].y : 0.f));
+            acc += ww[u] * (amv[u] == (zz[u] & 255) ? cgv[u].y : cgv[u].x);
         }
     };
     int4 ta, za, tb4, zb;
