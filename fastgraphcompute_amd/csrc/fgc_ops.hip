@@ -1,6 +1,5 @@
 // index_replacer, kNN gradient, select_with_default and the fused GravNet
 // neighbour aggregation (forward / backward).  gfx950, wave64.
-#include <atomic>
 #include "fgc_common.h"
 #include "fgc_internal.h"
 
@@ -1170,18 +1169,8 @@ extern "C" int fgc_gravnet_aggregate_bwd_sorted_f32(const int32_t *d_nbr_sorted,
     hipStream_t s = (hipStream_t)stream;
     const int pw = pick_pw(P);
     const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GT_WAVES * GT);
-    const size_t lds = gravnet_tile_lds(pw, K);
-    // more than 64 KB of dynamic LDS per block (P > 32 with K = 64) has to be granted per kernel, once
+    const size_t lds = gravnet_tile_lds(pw, K);          // at most 47 KB (P = K = 64)
 #define FGC_L(PWW)                                                                                              \
-    if (lds > 65536) {                                                                                          \
-        static std::atomic<size_t> granted{0};                                                                  \
-        if (granted.load() < lds) {                                                                             \
-            if (hipFuncSetAttribute((const void *)k_gravnet_bwd_tile<PWW>,                                      \
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)        \
-                return FGC_EUNSUPPORTED;                                                                        \
-            granted.store(lds);                                                                                 \
-        }                                                                                                       \
-    }                                                                                                           \
     hipLaunchKernelGGL((k_gravnet_bwd_tile<PWW>), dim3(blocks), dim3(GT_WAVES * 64), lds, s, d_nbr_sorted,      \
                        (const uint32_t *)d_order, d_distsq, d_feat, (int)ld_feat, d_argmax, d_grad_fmean,      \
                        d_grad_fmax, (int)ld_grad, d_grad_feat, (int)ld_grad_feat, d_grad_distsq, n_vert, (int)K, \

@@ -38,6 +38,9 @@ extern "C" {
 #define FGC_MAX_K 1024       /* neighbours per query the kNN kernels support; the reference's loops take any
                                 K (binned_select_knn_cpu.cpp:211-326), its benchmarks stop at 100.  Up to 256
                                 the search runs its register-tiled kernels, beyond that a slower variant  */
+#define FGC_MAX_VERTICES ((1ll << 31) - 65) /* points per call of the kNN entry points: sorted positions are 32-bit
+                                (FGC_EINVAL beyond); the reference indexes with int64 but its [N, K] int64 output
+                                alone is 1 TB at K = 64 there */
 /* bits of the kNN entry points' tf_compat argument */
 #define FGC_KNN_TF_COMPAT 1  /* padding slots name the query itself instead of -1 (binned_select_knn.py:7-9) */
 #define FGC_KNN_ANY_ORDER 2  /* slots 1.. of a row in any order instead of by increasing distance: the reference

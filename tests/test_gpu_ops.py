@@ -407,3 +407,70 @@ def test_gravnet_backward_in_sorted_space_rejects_unsupported_shapes():
     assert L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, 32, p, p, p, 32, p, 32, p, 100, 65, 32, None, None) == -3
     assert L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, 8, p, p, p, 8, p, 8, p, 100, 8, 8, None, None) == -3
     assert L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, 16, p, p, p, 32, p, 32, p, 100, 8, 32, None, None) == -1
+
+
+def test_out_of_range_neighbour_indices_are_flagged_not_followed(oracle):
+    """A neighbour index >= the number of points must not be dereferenced: every kernel that follows indices treats it
+    as an empty slot and sets FGC_ST_BAD_INDEX in the status word.  Through the C ABI, against the same call with
+    those entries set to -1."""
+    import ctypes
+    from fastgraphcompute_amd import _lib, _ops
+    L = _lib.lib()
+    n, S, K, P = 3000, 3, 24, 32
+    rng = np.random.default_rng(77)
+    space = torch.from_numpy((rng.standard_normal((n, S)) * 0.3).astype(np.float32)).cuda()
+    rs = torch.tensor([0, 1200, n], device="cuda")
+    idx, dist, nbr, order = _ops._knn_forward(space, S, rs, K, None, None, 3, False, True)
+    hit = torch.from_numpy(rng.random((n, K)) < 0.02).cuda()
+    hit[:, 0] = False
+    hit_sorted = hit[order.long()]                                   # the same pairs in the search's sorted rows
+    feat = torch.from_numpy(rng.standard_normal((n, P)).astype(np.float32)).cuda()
+    g = torch.from_numpy(rng.standard_normal((n, 2 * P)).astype(np.float32)).cuda()
+    gk = torch.from_numpy(rng.standard_normal((n, K)).astype(np.float32)).cuda()
+    st = _lib.stream_ptr()
+
+    def run(fill):
+        i2 = torch.where(hit, torch.full_like(idx, fill), idx)
+        # the search's sorted rows hold the slots of a row in the same order as the original rows
+        n2 = torch.where(hit_sorted, torch.full_like(nbr, fill), nbr)
+        res, flags = {}, {}
+        status = torch.zeros(4, dtype=torch.int32, device="cuda")
+        fm, fx = torch.empty((n, P), device="cuda"), torch.empty((n, P), device="cuda")
+        am = torch.empty((n, P), dtype=torch.int32, device="cuda")
+        _lib.check(L.fgc_gravnet_aggregate_fwd_ld_f32(_lib.ptr(i2), _lib.ptr(dist), _lib.ptr(feat), P, n, _lib.ptr(fm),
+                                                      _lib.ptr(fx), P, _lib.ptr(am), n, K, P, _lib.ptr(status), st))
+        torch.cuda.synchronize()
+        res["fwd"], flags["fwd"] = (fm.cpu().numpy(), fx.cpu().numpy()), int(status[0])
+        for name in ("pairs", "tiles"):
+            status.zero_()
+            gf, gd = torch.zeros((n, P), device="cuda"), torch.empty((n, K), device="cuda")
+            if name == "pairs":
+                rc = L.fgc_gravnet_aggregate_bwd_ld_f32(_lib.ptr(i2), _lib.ptr(dist), _lib.ptr(feat), P, n, _lib.ptr(am),
+                                                        _lib.ptr(g), ctypes.c_void_p(g.data_ptr() + 4 * P), 2 * P,
+                                                        _lib.ptr(gf), P, _lib.ptr(gd), n, K, P, _lib.ptr(status), st)
+            else:
+                rc = L.fgc_gravnet_aggregate_bwd_sorted_f32(_lib.ptr(n2), _lib.ptr(order), _lib.ptr(dist),
+                                                            _lib.ptr(feat), P, _lib.ptr(am), _lib.ptr(g),
+                                                            ctypes.c_void_p(g.data_ptr() + 4 * P), 2 * P, _lib.ptr(gf),
+                                                            P, _lib.ptr(gd), n, K, P, _lib.ptr(status), st)
+            _lib.check(rc)
+            torch.cuda.synchronize()
+            res[name], flags[name] = (gf.cpu().numpy(), gd.cpu().numpy()), int(status[0])
+        status.zero_()
+        gx = torch.empty((n, S), device="cuda")
+        _lib.check(L.fgc_binned_select_knn_grad_f32(_lib.ptr(gk), _lib.ptr(i2), _lib.ptr(space), _lib.ptr(gx), n, K, S,
+                                                    None, _lib.ptr(status), st))
+        torch.cuda.synchronize()
+        res["knn_grad"], flags["knn_grad"] = (gx.cpu().numpy(),), int(status[0])
+        return res, flags
+
+    want, clean = run(-1)
+    got, flagged = run(n + 5)
+    for name in want:
+        assert clean[name] & _lib.ST_BAD_INDEX == 0, name
+        assert flagged[name] & _lib.ST_BAD_INDEX, name
+        for a, b in zip(got[name], want[name]):
+            if name == "fwd":
+                np.testing.assert_array_equal(a, b, err_msg=name)
+            else:
+                assert _rel_err(a, b) < DIST_RTOL, name
