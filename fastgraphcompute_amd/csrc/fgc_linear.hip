@@ -90,15 +90,22 @@ __global__ __launch_bounds__(256) void k_linear_wgrad(const float *__restrict__ 
     }
 }
 
-// out[e] = sum over the splits of part[s * count + e].  A block owns 64 consecutive outputs; its four wavefronts
-// sum every fourth split (eight loads in flight) and the four sums are added in wavefront order: a fixed order,
-// so the result is reproducible.
-__global__ __launch_bounds__(256) void k_sum_partials(const float *__restrict__ part, int n_splits, int64_t count,
-                                                      float *__restrict__ out)
+// out[e] = sum over the splits of part[s * count + e], for two arrays in one launch (weights: blocks 0 .. blocks_a - 1,
+// bias: the blocks after them).  A block owns 64 consecutive outputs; its four wavefronts sum every fourth split
+// (eight loads in flight) and the four sums are added in wavefront order: a fixed order, so the result is
+// reproducible.
+__global__ __launch_bounds__(256) void k_sum_partials(const float *__restrict__ part_a, int64_t count_a,
+                                                      float *__restrict__ out_a, int blocks_a,
+                                                      const float *__restrict__ part_b, int64_t count_b,
+                                                      float *__restrict__ out_b, int n_splits)
 {
     __shared__ float s_sum[4][64];
     const int lane = fgc_lane(), w = threadIdx.x >> 6;
-    const int64_t e = (int64_t)blockIdx.x * 64 + lane;
+    const bool second = (int)blockIdx.x >= blocks_a;
+    const float *__restrict__ part = second ? part_b : part_a;
+    float *__restrict__ out = second ? out_b : out_a;
+    const int64_t count = second ? count_b : count_a;
+    const int64_t e = (int64_t)(second ? (int)blockIdx.x - blocks_a : (int)blockIdx.x) * 64 + lane;
     float acc[8];
 #pragma unroll
     for (int u = 0; u < 8; u++) acc[u] = 0.f;
@@ -177,13 +184,9 @@ extern "C" int fgc_linear_wgrad_f32(const float *d_grad_out, const float *d_inpu
                            p.groups_i, p.n_splits, p.pts_per_split, part_w, part_b);
     FGC_LAUNCH_CHECK();
     const int64_t cw = (int64_t)n_out * n_in;
-    hipLaunchKernelGGL(k_sum_partials, dim3((unsigned)fgc_cdiv(cw, 64)), block, 0, s, (const float *)part_w,
-                       p.n_splits, cw, d_grad_weight);
+    const int blocks_w = (int)fgc_cdiv(cw, 64), blocks_b = d_grad_bias ? (int)fgc_cdiv(n_out, 64) : 0;
+    hipLaunchKernelGGL(k_sum_partials, dim3((unsigned)(blocks_w + blocks_b)), block, 0, s, (const float *)part_w, cw,
+                       d_grad_weight, blocks_w, (const float *)part_b, (int64_t)n_out, d_grad_bias, p.n_splits);
     FGC_LAUNCH_CHECK();
-    if (d_grad_bias) {
-        hipLaunchKernelGGL(k_sum_partials, dim3((unsigned)fgc_cdiv(n_out, 64)), block, 0, s,
-                           (const float *)part_b, p.n_splits, (int64_t)n_out, d_grad_bias);
-        FGC_LAUNCH_CHECK();
-    }
     return FGC_OK;
 }
