@@ -11,7 +11,10 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["fgc_binning.hip", "fgc_knn.hip", "fgc_ops.hip", "fgc_oc.hip", "fgc_linear.hip", "fgc_api.hip"]
+# (source, object, extra flags): the search kernels are compiled a second time with their statistics counters
+SOURCES = [("fgc_binning.hip", "fgc_binning.o", []), ("fgc_knn.hip", "fgc_knn.o", []),
+           ("fgc_knn.hip", "fgc_knn_stats.o", ["-DFGC_KNN_STATS"]), ("fgc_ops.hip", "fgc_ops.o", []),
+           ("fgc_oc.hip", "fgc_oc.o", []), ("fgc_linear.hip", "fgc_linear.o", []), ("fgc_api.hip", "fgc_api.o", [])]
 OUT = os.path.join(os.path.dirname(HERE), "libfgc_hip.so")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
@@ -21,9 +24,9 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
 def build(verbose=True, extra=()):
     objs = []
     procs = []
-    for src in SOURCES:
-        obj = os.path.join(HERE, src.replace(".hip", ".o"))
-        cmd = ["hipcc"] + FLAGS + list(extra) + ["-c", os.path.join(HERE, src), "-o", obj]
+    for src, obj_name, more in SOURCES:
+        obj = os.path.join(HERE, obj_name)
+        cmd = ["hipcc"] + FLAGS + more + list(extra) + ["-c", os.path.join(HERE, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((subprocess.Popen(cmd), src))

@@ -215,7 +215,7 @@ int knn_search(float tau0, int32_t *d_nbr_sorted, int64_t n_vert, int32_t n_coor
     a.tau0 = tau0;
     a.out_sorted = d_nbr_sorted;
     a.out_idx = d_idx; a.out_dist = d_distsq; a.stats = (unsigned long long *)d_stats;
-    return fgc_launch_knn(a, (hipStream_t)stream);
+    return a.stats ? fgc_launch_knn_stats(a, (hipStream_t)stream) : fgc_launch_knn(a, (hipStream_t)stream);
 }
 
 extern "C" int fgc_binned_knn_export_order_i32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,

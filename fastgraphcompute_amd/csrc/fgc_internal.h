@@ -43,4 +43,5 @@ struct KnnArgs {
                                 // query, entries = sorted positions), for the gradient kernel
     unsigned long long *stats;  // optional counters
 };
-int fgc_launch_knn(const KnnArgs &a, hipStream_t s);
+int fgc_launch_knn(const KnnArgs &a, hipStream_t s);        // a.stats is ignored
+int fgc_launch_knn_stats(const KnnArgs &a, hipStream_t s);  // the same search, counting into a.stats (slower)

@@ -41,6 +41,17 @@
 #include "fgc_common.h"
 #include "fgc_internal.h"
 
+// This file is compiled twice: as it is, and with -DFGC_KNN_STATS for the variant that also counts distance
+// evaluations, candidate chunks and prunes (fgc_launch_knn_stats, kernels k_knn_stats): the counters cost scalar
+// registers and instructions in the inner loops (3-5 % of the search), so calls that do not ask for them get
+// kernels without.
+#ifdef FGC_KNN_STATS
+#define k_knn k_knn_stats
+#define fgc_launch_knn fgc_launch_knn_stats
+#elif defined(FGC_KNN_COUNTERS)
+#error "the debug counters need the statistics build (-DFGC_KNN_STATS)"
+#endif
+
 #ifndef QT
 #define QT 6           // queries per wavefront (6 x 128 pool slots x 8 B = 6 KB of LDS at K = 64: 26 wavefronts per CU)
 #endif
@@ -192,8 +203,10 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     bool qactive = isq;
     if (a.sdir && isq) { unsigned char dd = a.sdir[qs]; qactive = !(dd == 0 || dd == 2); }
 
+#ifdef FGC_KNN_STATS
     unsigned long long nev = 0;
     unsigned nchunks = 0, nprunes = 0;
+#endif
 #ifdef FGC_KNN_COUNTERS
     unsigned n_cullq = 0, n_app = 0, n_span = 0, n_bis = 0, n_bisx = 0;
 #define CNT(x) x
@@ -290,7 +303,9 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             }
             base += __popcll(km);
         }
+#ifdef FGC_KNN_STATS
         nprunes++;
+#endif
         const float tnew = __uint_as_float(hi);
         tau = (lane == q) ? tnew : tau;
         cnt = (lane == q) ? newc : cnt;
@@ -373,7 +388,9 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 #pragma unroll
                 for (int dd = 0; dd < DR; dd++) sx[s][dd] = (ra + s <= rb && dd < a.D) ? sc[(size_t)dd * ldc + j] : 0.f;
             }
+#ifdef FGC_KNN_STATS
             nchunks += (unsigned)(rb - ra + 1);
+#endif
             for (unsigned long long m = gm; m;) {
                 const int q = __ffsll((long long)m) - 1;
                 m &= m - 1;
@@ -391,7 +408,9 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     ds[s] = ok ? __float_as_uint(dsq) : 0xffffffffu;
                     const unsigned long long okm = fgc_ballot(ok);
                     total += __popcll(okm);
+#ifdef FGC_KNN_STATS
                     nev += (unsigned long long)__popcll(fgc_ballot(sv[s]));
+#endif
                     mx = max(mx, ok ? ds[s] : 0u);
                 }
                 unsigned sel = 0xfffffffeu;             // candidates <= sel are pushed: everything by default
@@ -621,8 +640,10 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     bool cand_ok = v;
                     if (a.sdir && v) { unsigned char dd = a.sdir[j]; if (dd == 1 || dd == 2) cand_ok = false; }
                     if (DT > 0 && !cand_ok) cx[0] = INFINITY;
+#ifdef FGC_KNN_STATS
                     nev += (unsigned long long)__popcll(cact) * (unsigned)(min(j1, base + 64) - max(j0, base));
                     nchunks++;
+#endif
                     for (unsigned long long m = cact; m;) {
                         const int q = __ffsll((long long)m) - 1;
                         m &= m - 1;
@@ -739,6 +760,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             }
         }
     }
+#ifdef FGC_KNN_STATS
     if (a.stats && lane == 0) {
 #ifdef FGC_KNN_COUNTERS
         atomicAdd(&a.stats[3], (unsigned long long)n_cullq); atomicAdd(&a.stats[4], (unsigned long long)n_app);
@@ -749,6 +771,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
         atomicAdd(&a.stats[1], (unsigned long long)nchunks);
         atomicAdd(&a.stats[2], (unsigned long long)nprunes);
     }
+#endif
 }
 
 template <int DT, int NSEG, int RD> static int launch_knn_t(const KnnArgs &a, hipStream_t s)
