@@ -49,7 +49,7 @@
 #define k_knn k_knn_stats
 #define fgc_launch_knn fgc_launch_knn_stats
 #elif defined(FGC_KNN_COUNTERS)
-#error "the debug counters need the statistics build (-DFGC_KNN_STATS)"
+#undef FGC_KNN_COUNTERS        // the debug counters exist in the statistics build only
 #endif
 
 #ifndef QT
