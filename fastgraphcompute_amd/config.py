@@ -21,6 +21,6 @@ tile_aggregation_backward = True
 
 # binned_select_knn returns a row's neighbours (slots 1.., after the query itself in slot 0) in no particular order,
 # as the reference does (its kernel replaces the farthest entry in place; its tests sort each row before comparing).
-# True: by increasing distance, at the price of a per-query sort inside the search kernel (+9 % at 1 M points, K = 64).
+# True: by increasing distance, at the price of a per-query sort inside the search kernel (+10 % at 1 M points, K = 64).
 # The neighbour set, the distances and the gradients are the same either way.
 sorted_neighbours = False
