@@ -6,7 +6,8 @@
 sync_checks = True
 
 # Accumulate the kNN kernel's counters (distance evaluations, candidate chunks,
-# pool prunes) into binned_select_knn.last_stats; used by the benchmark.
+# pool prunes) into binned_select_knn.last_stats; used by the benchmark.  Calls that collect them run the
+# statistics build of the search kernels, which is slower (counters in the inner loops, one atomic per wavefront).
 collect_stats = False
 
 # When binned_select_knn is called without n_bins, size the search grid for this library's search (coarse bins

@@ -130,7 +130,9 @@ int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t ld_coords,
  *   d_stats       optional uint64[8] device counters, accumulated: [0] distance
  *                 evaluations, [1] candidate chunks visited, [2] pool prunes
  *                 ([3..7] only in debug builds with -DFGC_KNN_COUNTERS: box
- *                 tests, appends, spans, bisection steps); NULL to skip
+ *                 tests, appends, spans, bisection steps); NULL to skip.  A call
+ *                 with d_stats runs a second build of the search kernels that carries
+ *                 the counters and is slower (time a call without)
  */
 size_t fgc_binned_select_knn_workspace_bytes(int64_t n_vert, int32_t n_coords,
                                              int32_t n_bin_dims, const int64_t *n_bins,
