@@ -388,3 +388,25 @@ def test_two_host_threads_on_their_own_streams():
     torch.cuda.synchronize()
     assert out["good_err"] == [] and out["good_ok"] == 25, out
     assert out["bad_other"] == [] and out["bad_raised"] == 25, out
+
+
+def test_statistics_build_returns_the_same_rows():
+    """A call that asks for the search counters runs a second build of the search kernels (with the counters in
+    its inner loops): rows and distances must be identical to the plain build's, and the counters plausible."""
+    from fastgraphcompute_amd import binned_select_knn, config
+    rng = np.random.default_rng(31)
+    for D, K in ((3, 16), (4, 40), (8, 100)):
+        n = 6000
+        coords = torch.from_numpy(rng.standard_normal((n, D)).astype(np.float32)).cuda()
+        rs = torch.tensor([0, 2500, n], device="cuda")
+        i0, d0 = binned_select_knn(K, coords, rs)
+        config.collect_stats = True
+        try:
+            i1, d1 = binned_select_knn(K, coords, rs)
+        finally:
+            config.collect_stats = False
+        assert torch.equal(i0, i1) and torch.equal(d0, d1)
+        from fastgraphcompute_amd import _ops
+        st = _ops.last_stats
+        assert st["n_vert"] == n and st["K"] == K
+        assert st["distance_evaluations"] >= n * min(K, 2500 - 1) and st["candidate_chunks"] > 0
