@@ -169,7 +169,11 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     const int nq = min(QT, a.n - qbeg);
     uint2 *pool = s_pool + (size_t)wv * QT * CAP;
 
-    const int K = a.K, nbd = a.nbd, ldc = a.ldc, nch = a.n_chunks;
+    const int K = a.K, ldc = a.ldc, nch = a.n_chunks;
+    const int nbd = RD >= 2 ? RD + 1 : a.nbd;     // binned dimensions: RD + 1 except for the smallest instantiation (1 or 2)
+    // coordinates per point: a compile-time constant where the kernel is built for exactly that many (2 .. 8), so
+    // that the per-coordinate guards of the loads fold away
+    const int Dn = (DT >= 2 && DT <= 8) ? DT : a.D;
     const float *__restrict__ sc = a.sc;
     const int *__restrict__ bb = a.bb;
 
@@ -191,7 +195,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     float qx[DR];
     if (DT > 0) {
 #pragma unroll
-        for (int d = 0; d < DR; d++) qx[d] = (d < a.D) ? sc[(size_t)d * ldc + qs] : 0.f;   // padded dimensions: 0
+        for (int d = 0; d < DR; d++) qx[d] = (d < Dn) ? sc[(size_t)d * ldc + qs] : 0.f;   // padded dimensions: 0
     }
     float qb[RD];  // normalised row-dimension coordinates
 #pragma unroll
@@ -327,6 +331,16 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
         if (!pm) return;
         CNT(n_app++);
         int pc = fgc_readlane_i(cnt, q);
+        {
+            // the common case on a short path of its own: everything fits with room to spare and the query has
+            // a bound already (what the loop below does in its first pass when it ends there)
+            const int pn = pc + __popcll(pm);
+            if (pn <= CAP - PRUNE_MARGIN && (pn <= K || ((fgc_ballot(tau < INFINITY) >> q) & 1ull))) {
+                if (want) pool[q * CAP + pc + fgc_mbcnt(pm)] = make_uint2(__float_as_uint(dsq), (unsigned)j);
+                cnt = (lane == q) ? pn : cnt;
+                return;
+            }
+        }
         for (int attempt = 0;; attempt++) {
             const int room = CAP - pc;
             const int rnk = fgc_mbcnt(pm);
@@ -386,7 +400,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                 sv[s] = (ra + s <= rb) && j >= ev_j0 && j < ev_j1;
                 if (a.sdir && sv[s]) { unsigned char dd = a.sdir[j]; if (dd == 1 || dd == 2) sv[s] = false; }
 #pragma unroll
-                for (int dd = 0; dd < DR; dd++) sx[s][dd] = (ra + s <= rb && dd < a.D) ? sc[(size_t)dd * ldc + j] : 0.f;
+                for (int dd = 0; dd < DR; dd++) sx[s][dd] = (ra + s <= rb && dd < Dn) ? sc[(size_t)dd * ldc + j] : 0.f;
             }
 #ifdef FGC_KNN_STATS
             nchunks += (unsigned)(rb - ra + 1);
@@ -571,7 +585,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     float g2 = g * g;
 #pragma unroll
                     for (int dd = 1; dd < DR; dd++) {
-                        if (dd < a.D) {
+                        if (dd < Dn) {
                             g = fmaxf(fmaxf(a.sbox_lo[(size_t)dd * a.n_super + sb] - qx[dd],
                                             qx[dd] - a.sbox_hi[(size_t)dd * a.n_super + sb]), 0.f);
                             g2 += g * g;
@@ -588,8 +602,8 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     float blo[DR], bhi[DR];
 #pragma unroll
                     for (int dd = 0; dd < DR; dd++) {
-                        blo[dd] = (cv && dd < a.D) ? a.box_lo[(size_t)dd * nch + c] : 0.f;
-                        bhi[dd] = (cv && dd < a.D) ? a.box_hi[(size_t)dd * nch + c] : 0.f;
+                        blo[dd] = (cv && dd < Dn) ? a.box_lo[(size_t)dd * nch + c] : 0.f;
+                        bhi[dd] = (cv && dd < Dn) ? a.box_hi[(size_t)dd * nch + c] : 0.f;
                     }
                     mymask = 0u;
                     for (unsigned long long m = actb; m;) {
@@ -617,7 +631,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                 if (DT > 0 && any) {
                     const int jn = ((cb + __ffsll((long long)any) - 1) << 6) + lane;
 #pragma unroll
-                    for (int dd = 0; dd < DR; dd++) nx[dd] = (dd < a.D) ? sc[(size_t)dd * ldc + jn] : 0.f;
+                    for (int dd = 0; dd < DR; dd++) nx[dd] = (dd < Dn) ? sc[(size_t)dd * ldc + jn] : 0.f;
                 }
                 while (any) {
                     const int l = __ffsll((long long)any) - 1;
@@ -634,7 +648,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                         if (any) {
                             const int jn = ((cb + __ffsll((long long)any) - 1) << 6) + lane;
 #pragma unroll
-                            for (int dd = 0; dd < DR; dd++) nx[dd] = (dd < a.D) ? sc[(size_t)dd * ldc + jn] : 0.f;
+                            for (int dd = 0; dd < DR; dd++) nx[dd] = (dd < Dn) ? sc[(size_t)dd * ldc + jn] : 0.f;
                         }
                     }
                     bool cand_ok = v;
@@ -659,7 +673,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                             if (cand_ok) {
                                 float df = sc[qbeg + q] - sc[j];
                                 dsq = df * df;
-                                for (int dd = 1; dd < a.D; dd++) {
+                                for (int dd = 1; dd < Dn; dd++) {
                                     df = sc[(size_t)dd * ldc + qbeg + q] - sc[(size_t)dd * ldc + j];
                                     dsq += df * df;
                                 }
