@@ -309,7 +309,8 @@ def _knn_forward(coords: torch.Tensor, D: int, row_splits, K: int, direction, n_
                 nbr_sorted = torch.empty((n, K), dtype=torch.int32, device=dev)
             _lib.check(L.fgc_binned_knn_search_f32(
                 n, D, rs_arr, n_rs, K, nbd, nb_arr, 1 if dirt is not None else 0,
-                (_lib.KNN_TF_COMPAT if tf_compat else 0) | (0 if config.sorted_neighbours else _lib.KNN_ANY_ORDER),
+                (_lib.KNN_TF_COMPAT if tf_compat else 0) | (0 if config.sorted_neighbours else _lib.KNN_ANY_ORDER)
+                | (0 if config.matrix_search else _lib.KNN_NO_MATRIX),
                 _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(nbr_sorted), _lib.ptr(stats), _lib.ptr(ws), ws_bytes, st))
             if want_backward:
                 order = torch.empty(n, dtype=torch.int32, device=dev)

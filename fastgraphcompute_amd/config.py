@@ -25,3 +25,8 @@ tile_aggregation_backward = True
 # True: by increasing distance, at the price of a per-query sort inside the search kernel (+10 % at 1 M points, K = 64).
 # The neighbour set, the distances and the gradients are the same either way.
 sorted_neighbours = False
+
+# Searches over points with 5 to 8 coordinates (K <= 256) screen their candidates on the matrix cores and compute exact
+# distances only for the pairs that can still matter.  False: the vector-unit search, as for every other shape.  Same
+# neighbours and bit-identical distances either way.
+matrix_search = True

@@ -13,7 +13,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 # (source, object, extra flags): the search kernels are compiled a second time with their statistics counters
 SOURCES = [("fgc_binning.hip", "fgc_binning.o", []), ("fgc_knn.hip", "fgc_knn.o", []),
-           ("fgc_knn.hip", "fgc_knn_stats.o", ["-DFGC_KNN_STATS"]), ("fgc_ops.hip", "fgc_ops.o", []),
+           ("fgc_knn.hip", "fgc_knn_stats.o", ["-DFGC_KNN_STATS"]),
+           ("fgc_knn_mfma.hip", "fgc_knn_mfma.o", ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]), ("fgc_ops.hip", "fgc_ops.o", []),
            ("fgc_oc.hip", "fgc_oc.o", []), ("fgc_linear.hip", "fgc_linear.o", []), ("fgc_api.hip", "fgc_api.o", [])]
 OUT = os.path.join(os.path.dirname(HERE), "libfgc_hip.so")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",

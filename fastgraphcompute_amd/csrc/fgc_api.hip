@@ -24,7 +24,8 @@ extern "C" const char *fgc_error_string(int code)
 
 namespace {
 struct KnnWorkspace {
-    size_t geom, partial, keys, vals, sort, sort_alt_vals, bb, sc, sdir, box_lo, box_hi, sbox_lo, sbox_hi, total;
+    size_t geom, partial, keys, vals, sort, sort_alt_vals, bb, sc, sp, redo, sdir, box_lo, box_hi, sbox_lo, sbox_hi, total;
+    bool with_sp;
     int ldc;
 };
 
@@ -39,7 +40,7 @@ int64_t total_bins(int n_bin_dims, const int64_t *n_bins, int n_rs)
     return b;
 }
 
-KnnWorkspace plan(int64_t n, int D, int nbd, const int64_t *n_bins, int n_rs, bool with_dir)
+KnnWorkspace plan(int64_t n, int D, int K, int nbd, const int64_t *n_bins, int n_rs, bool with_dir)
 {
     KnnWorkspace w;
     size_t off = 0;
@@ -55,6 +56,9 @@ KnnWorkspace plan(int64_t n, int D, int nbd, const int64_t *n_bins, int n_rs, bo
     w.sort_alt_vals = fgc_align((size_t)n * 4);  // offset of the alternate value buffer inside the sort area
     w.bb = take((size_t)(B + 1) * 4);
     w.sc = take((size_t)w.ldc * D * 4);
+    w.with_sp = fgc_knn_uses_mfma(D, K);     // rows of 8 floats for the matrix-core search
+    w.sp = take(w.with_sp ? (size_t)w.ldc * 32 : 0);
+    w.redo = take(w.with_sp ? (size_t)w.ldc : 0);   // flags of the queries the matrix-core search leaves to the vector search
     w.sdir = take(with_dir ? (size_t)n : 0);
     w.box_lo = take((size_t)(w.ldc / 64) * D * 4);
     w.box_hi = take((size_t)(w.ldc / 64) * D * 4);
@@ -68,9 +72,8 @@ KnnWorkspace plan(int64_t n, int D, int nbd, const int64_t *n_bins, int n_rs, bo
 extern "C" size_t fgc_binned_select_knn_workspace_bytes(int64_t n_vert, int32_t n_coords, int32_t n_bin_dims,
                                                         const int64_t *n_bins, int32_t n_rs, int32_t K)
 {
-    (void)K;
     if (n_vert <= 0 || !n_bins || n_bin_dims < 1 || n_bin_dims > FGC_MAX_BIN_DIMS) return 256;
-    return plan(n_vert, n_coords, n_bin_dims, n_bins, n_rs, true).total;
+    return plan(n_vert, n_coords, K, n_bin_dims, n_bins, n_rs, true).total;
 }
 
 namespace {
@@ -112,7 +115,7 @@ int knn_validate(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_hos
         if (row_splits_host[r] < row_splits_host[r - 1]) return FGC_EINVAL;
     c->B = total_bins(n_bin_dims, n_bins, n_rs);
     if (c->B < 0 || c->B >= (1ll << 31)) return FGC_EINVAL;
-    c->w = plan(n_vert > 0 ? n_vert : 1, n_coords, n_bin_dims, n_bins, n_rs, with_dir);
+    c->w = plan(n_vert > 0 ? n_vert : 1, n_coords, K, n_bin_dims, n_bins, n_rs, with_dir);
     int bin_bits = 1;
     while ((1ll << bin_bits) < c->B) bin_bits++;
     c->sub_bits = choose_sub_bits(bin_bits, n_bin_dims);
@@ -179,7 +182,8 @@ extern "C" int fgc_binned_knn_prepare_ld_f32(const float *d_coords, int64_t n_ve
     if (skeys2 != skeys || order2 != order) return FGC_EINVAL;  // internal layout mismatch
     rc = fgc_launch_bin_boundaries(skeys, (int)n_vert, c.sub_bits * n_bin_dims, (int)c.B, bb, s);
     if (rc) return rc;
-    rc = fgc_launch_gather_sorted(d_coords, ld_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir, s);
+    rc = fgc_launch_gather_sorted(d_coords, ld_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir,
+                                  w.with_sp ? (float *)(ws + w.sp) : nullptr, fgc_knn_sp_half(n_coords), s);
     if (rc) return rc;
     return fgc_launch_chunk_boxes(sc, (int)n_vert, n_coords, w.ldc, (float *)(ws + w.box_lo),
                                   (float *)(ws + w.box_hi), (float *)(ws + w.sbox_lo), (float *)(ws + w.sbox_hi), s);
@@ -215,6 +219,14 @@ int knn_search(float tau0, int32_t *d_nbr_sorted, int64_t n_vert, int32_t n_coor
     a.tau0 = tau0;
     a.out_sorted = d_nbr_sorted;
     a.out_idx = d_idx; a.out_dist = d_distsq; a.stats = (unsigned long long *)d_stats;
+    a.sp = c.w.with_sp ? (const float *)(ws + c.w.sp) : nullptr;
+    a.redo = nullptr;
+    // many coordinates: candidates screened on the matrix cores (a radius bound keeps the vector search, which
+    // culls by it from the first bin row on)
+    if (a.sp && !(tf_compat & FGC_KNN_NO_MATRIX) && !(tau0 < INFINITY)) {
+        a.redo = (unsigned char *)(ws + c.w.redo);
+        return a.stats ? fgc_launch_knn_mfma_stats(a, (hipStream_t)stream) : fgc_launch_knn_mfma(a, (hipStream_t)stream);
+    }
     return a.stats ? fgc_launch_knn_stats(a, (hipStream_t)stream) : fgc_launch_knn(a, (hipStream_t)stream);
 }
 
@@ -321,7 +333,7 @@ extern "C" int fgc_binned_select_knn_noalloc_f32(const float *d_coords, int64_t 
 {
     if (n_vert < 0 || n_coords < 1 || n_rs < 2 || !n_bins || n_bin_dims < 1 || n_bin_dims > FGC_MAX_BIN_DIMS)
         return FGC_EINVAL;
-    const size_t need = n_vert > 0 ? plan(n_vert, n_coords, n_bin_dims, n_bins, n_rs, d_direction != nullptr).total : 0;
+    const size_t need = n_vert > 0 ? plan(n_vert, n_coords, K, n_bin_dims, n_bins, n_rs, d_direction != nullptr).total : 0;
     if (need > (size_t)FGC_NOALLOC_SCRATCH_BYTES) return FGC_ETOOLARGE;
     void *ws = nullptr;
     int rc = scratch_address(&ws);

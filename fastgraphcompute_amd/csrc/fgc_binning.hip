@@ -617,12 +617,28 @@ __global__ __launch_bounds__(256) void k_gather_sorted(const float *__restrict__
                                                        const uint32_t *__restrict__ order, int n, int D,
                                                        int ldc, float *__restrict__ sc,
                                                        const int64_t *__restrict__ direction,
-                                                       unsigned char *__restrict__ sdir)
+                                                       unsigned char *__restrict__ sdir, float4 *__restrict__ sp,
+                                                       int sp_half)
 {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (sp && i >= n && i < ldc) {           // padding rows of the last chunk
+        sp[(int64_t)i * 2] = make_float4(0.f, 0.f, 0.f, 0.f);
+        sp[(int64_t)i * 2 + 1] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     if (i >= n) return;
     uint32_t o = order[i];
-    for (int d = 0; d < D; d++) sc[(int64_t)d * ldc + i] = coords[(int64_t)o * ld_in + d];
+    if (sp) {
+        float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int d = 0; d < D; d++) {
+            const float x = coords[(int64_t)o * ld_in + d];
+            sc[(int64_t)d * ldc + i] = x;
+            if (d < 2 * sp_half) r[d < sp_half ? d : 4 + d - sp_half] = x;
+        }
+        sp[(int64_t)i * 2] = make_float4(r[0], r[1], r[2], r[3]);
+        sp[(int64_t)i * 2 + 1] = make_float4(r[4], r[5], r[6], r[7]);
+    } else {
+        for (int d = 0; d < D; d++) sc[(int64_t)d * ldc + i] = coords[(int64_t)o * ld_in + d];
+    }
     if (sdir) {
         int64_t v = direction[o];
         sdir[i] = (unsigned char)((v >= 0 && v <= 2) ? v : 3);
@@ -647,10 +663,10 @@ int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int shift, int n_bin
 }
 
 int fgc_launch_gather_sorted(const float *coords, int ld_in, const uint32_t *order, int n, int D, int ldc, float *sc,
-                             const int64_t *direction, unsigned char *sdir, hipStream_t s)
+                             const int64_t *direction, unsigned char *sdir, float *sp, int sp_half, hipStream_t s)
 {
-    hipLaunchKernelGGL(k_gather_sorted, dim3((unsigned)fgc_cdiv(n, 256)), dim3(256), 0, s, coords, ld_in, order,
-                       n, D, ldc, sc, direction, sdir);
+    hipLaunchKernelGGL(k_gather_sorted, dim3((unsigned)fgc_cdiv(sp ? ldc : n, 256)), dim3(256), 0, s, coords, ld_in,
+                       order, n, D, ldc, sc, direction, sdir, (float4 *)sp, sp_half);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }

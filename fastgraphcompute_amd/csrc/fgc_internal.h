@@ -10,13 +10,16 @@ int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, int sub_b
 int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int shift, int n_bins_total, int *bb, hipStream_t s);
 int fgc_launch_chunk_boxes(const float *sc, int n, int D, int ldc, float *box_lo, float *box_hi, float *sbox_lo,
                            float *sbox_hi, hipStream_t s);
+// sp (optional): the sorted points once more as rows of 8 floats, two halves of 4 with `sp_half` coordinates each
+// (zero padded; rows n .. ldc - 1 are zero), for the matrix-core search
 int fgc_launch_gather_sorted(const float *coords, int ld_in, const uint32_t *order, int n, int D, int ldc, float *sc,
-                             const int64_t *direction, unsigned char *sdir, hipStream_t s);
+                             const int64_t *direction, unsigned char *sdir, float *sp, int sp_half, hipStream_t s);
 
 // kNN search over bin-sorted points (fgc_knn.hip)
 struct KnnArgs {
     const float *sc;            // sorted coordinates, structure of arrays [D][ldc]
     int ldc;
+    const float *sp;            // sorted coordinates as rows of 8 floats (matrix-core search only), or NULL
     const uint32_t *skeys;      // sorted key per point: (flat bin << key_shift) | Hilbert index inside the bin
     int key_shift;
     const float *box_lo;        // per 64-point chunk bounding boxes [D][n_chunks]
@@ -42,6 +45,15 @@ struct KnnArgs {
     int *out_sorted;            // optional [n, K]: the same rows in sorted space (row = sorted position of the
                                 // query, entries = sorted positions), for the gradient kernel
     unsigned long long *stats;  // optional counters
+    unsigned char *redo;        // NULL, or one flag per sorted position: the matrix-core search sets the flags of the
+                                // queries it leaves out, and the vector search then handles the flagged queries only
 };
 int fgc_launch_knn(const KnnArgs &a, hipStream_t s);        // a.stats is ignored
 int fgc_launch_knn_stats(const KnnArgs &a, hipStream_t s);  // the same search, counting into a.stats (slower)
+
+// kNN search with the candidates screened on the matrix cores (fgc_knn_mfma.hip): 5 to 8 coordinates, K <= 256,
+// needs a.sp.  Same rows as fgc_launch_knn up to the order inside a row and the choice between exactly tied candidates.
+bool fgc_knn_uses_mfma(int D, int K);
+inline int fgc_knn_sp_half(int D) { return D <= 6 ? 3 : 4; }   // coordinates per half row of sp
+int fgc_launch_knn_mfma(const KnnArgs &a, hipStream_t s);
+int fgc_launch_knn_mfma_stats(const KnnArgs &a, hipStream_t s);

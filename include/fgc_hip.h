@@ -47,6 +47,8 @@ extern "C" {
                                 promises no order either (its kernel replaces the farthest entry in place, its tests
                                 sort every row before comparing, tests/test_binned_select_knn.py:90-91); saves the
                                 per-query sort */
+#define FGC_KNN_NO_MATRIX 4  /* keep the vector-unit search where the library would screen the candidates on the
+                                matrix cores (5 to 8 coordinates, K <= 256); same neighbours, for comparison runs */
 
 #define FGC_STATUS_WORDS 4
 /* bits of d_status[0] */
@@ -120,7 +122,8 @@ int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t ld_coords,
  *                 :67-82) or passes the user's n_bins
  *   d_direction   int64 [n_vert] or NULL (0: only neighbour, 1: only query,
  *                 2: neither; binned_select_knn_cuda_kernel.cu:120-122,194-196)
- *   tf_compat     bit set of FGC_KNN_TF_COMPAT and FGC_KNN_ANY_ORDER (0 or 1 as before: rows by distance)
+ *   tf_compat     bit set of FGC_KNN_TF_COMPAT, FGC_KNN_ANY_ORDER and FGC_KNN_NO_MATRIX (0 or 1 as before: rows
+ *                 by distance)
  *   d_idx         out int64 [n_vert, K]: slot 0 the query itself, then its
  *                 K-1 nearest points of the same event by increasing distance
  *                 (in any order with FGC_KNN_ANY_ORDER), then -1 (or the
