@@ -89,6 +89,9 @@ def main():
     ap.add_argument("--cpu-reference-full", action="store_true",
                     help="also time the reference's own compiled CPU kernel (oracle/_ref) on ALL queries of the "
                          "workload, one core; minutes at the default workload")
+    ap.add_argument("--matrix-search", default="auto", choices=["auto", "off", "always"],
+                    help="config.matrix_search: let the library decide whether a search with 5 to 8 coordinates screens "
+                         "its candidates on the matrix cores (auto), never, or wherever that search can run")
     ap.add_argument("--sorted-neighbours", action="store_true",
                     help="ask for neighbour rows by increasing distance (config.sorted_neighbours) instead of the "
                          "default, rows in the order the search found them, as the reference returns them")
@@ -113,6 +116,7 @@ def main():
     torch.cuda.set_device(dev)
     L = _lib.lib()
     config.sorted_neighbours = bool(args.sorted_neighbours)
+    config.matrix_search = {"auto": True, "off": False, "always": "always"}[args.matrix_search]
 
     if args.workload == "oc_helper":
         print(json.dumps(oc_helper_workload(args, dev)), flush=True)
@@ -173,6 +177,7 @@ def main():
     nbr_sorted = torch.empty((n, K), dtype=torch.int32, device=dev)   # as the autograd path requests it
     st = _lib.stream_ptr()
     knn_flags = 0 if config.sorted_neighbours else _lib.KNN_ANY_ORDER     # the row order binned_select_knn asks for
+    knn_flags |= {"auto": 0, "off": _lib.KNN_NO_MATRIX, "always": _lib.KNN_FORCE_MATRIX}[args.matrix_search]
 
     def prepare():
         _lib.check(L.fgc_binned_knn_prepare_f32(_lib.ptr(coords), n, D, _lib.ptr(rs), rs_arr, n_rs, K, nbd, nb_arr,
@@ -198,6 +203,8 @@ def main():
     c_eval = int(stats[0].item())
     chunks = int(stats[1].item())
     inserts = int(stats[2].item())
+    handed_over, collected = int(stats[3].item()), int(stats[5].item())
+    matrix = collected > 0          # the search ran on the matrix cores (k_knn_mf); k_knn only took what it handed over
     reps = max(3, args.steps)
     t_prep = float(np.mean(timed(prepare, reps)))
     t_knn = float(np.mean(timed(lambda: search(False), reps)))
@@ -210,12 +217,24 @@ def main():
     # D-float candidate, every query is read once, every (idx, distsq) slot written once
     facts = profile_facts() if args.scale == 1.0 else {}
     clock_hz = GPU_CLOCK_HZ
-    bytes_alg = 4.0 * D * c_eval + 4.0 * D * n + 12.0 * K * n
+    # (the matrix-core search screens pairs in float16 and evaluates exact distances only for the candidates it collects:
+    # those are its distance evaluations; the screened pairs are reported separately)
+    n_exact = collected if matrix else c_eval
+    bytes_alg = 4.0 * D * n_exact + 4.0 * D * n + 12.0 * K * n
     # VALU wavefront instructions that are distance arithmetic: per 64 evaluations D subtractions, D
     # multiplications, D - 1 additions, the compare, and the D + 1 broadcasts of the query and its bound
-    roofline = roofline_entry("k_knn", w["name"], bytes_alg, t_knn, clock_hz, (c_eval / 64.0) * (4 * D + 1), facts)
+    roofline = roofline_entry("k_knn_mf" if matrix else "k_knn", w["name"], bytes_alg, t_knn, clock_hz,
+                              None if matrix else (c_eval / 64.0) * (4 * D + 1), facts)
+    if matrix:
+        # one v_mfma_f32_32x32x16_f16 per 32 x 32 pairs: 32 flops per evaluated pair, against the dense float16 peak
+        roofline["screened_pairs"] = c_eval
+        roofline["binding_resource"] = "valu_issue (histogram and collection of the screened pairs)"
+        roofline["matrix_core"] = {"mfma_tflops": round(32.0 * c_eval / (t_knn * 1e-3) / 1e12, 1), "peak_tflops": 2500.0,
+                                   "frac": round(32.0 * c_eval / (t_knn * 1e-3) / 1e12 / 2500.0, 4),
+                                   "candidates_collected_per_query": round(collected / max(1, n - handed_over), 1),
+                                   "queries_handed_to_the_vector_search": handed_over}
     achieved = roofline["achieved"]
-    roofline["distance_evaluations"] = c_eval
+    roofline["distance_evaluations"] = n_exact
     # inputs + outputs of the timed launch: queries, int64 indices, distances, int32 sorted-space rows
     roofline["io_floor_bytes"] = 4.0 * D * n + 16.0 * K * n
     # gradient kernel: upstream gradient + neighbour rows + one D-float gather per pair + coordinates in, gradient out
@@ -245,7 +264,8 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": w["name"], "n_points": n, "n_coords": D, "K": K, "events": int(n_rs - 1),
                    "n_bins": nb, "step": "binned_select_knn forward (whole call) + gradient",
-                   "row_order": "by distance" if config.sorted_neighbours else "any (as the reference)"},
+                   "row_order": "by distance" if config.sorted_neighbours else "any (as the reference)",
+                   "search_kernel": "k_knn_mf (candidates screened on the matrix cores)" if matrix else "k_knn"},
         "neighbours_per_s": round(n * K / t_step, 1),
         "forward_call_ms": round(t_prep + t_knn, 4),
         "forward_queries_per_s": round(n / ((t_prep + t_knn) * 1e-3), 1),

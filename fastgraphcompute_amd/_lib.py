@@ -66,7 +66,7 @@ SIGNATURES = {
 }
 
 ST_NONFINITE, ST_CLAMPED, ST_BAD_RANGE, ST_BAD_INDEX, ST_OC_TRUNCATED = 1, 2, 4, 8, 16
-KNN_TF_COMPAT, KNN_ANY_ORDER, KNN_NO_MATRIX = 1, 2, 4      # bits of the kNN entry points' tf_compat argument
+KNN_TF_COMPAT, KNN_ANY_ORDER, KNN_NO_MATRIX, KNN_FORCE_MATRIX = 1, 2, 4, 8   # bits of the kNN entry points' tf_compat argument
 
 
 def lib():

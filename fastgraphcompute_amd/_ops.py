@@ -310,7 +310,8 @@ def _knn_forward(coords: torch.Tensor, D: int, row_splits, K: int, direction, n_
             _lib.check(L.fgc_binned_knn_search_f32(
                 n, D, rs_arr, n_rs, K, nbd, nb_arr, 1 if dirt is not None else 0,
                 (_lib.KNN_TF_COMPAT if tf_compat else 0) | (0 if config.sorted_neighbours else _lib.KNN_ANY_ORDER)
-                | (0 if config.matrix_search else _lib.KNN_NO_MATRIX),
+                | (_lib.KNN_FORCE_MATRIX if config.matrix_search == "always" else
+                   (0 if config.matrix_search else _lib.KNN_NO_MATRIX)),
                 _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(nbr_sorted), _lib.ptr(stats), _lib.ptr(ws), ws_bytes, st))
             if want_backward:
                 order = torch.empty(n, dtype=torch.int32, device=dev)
@@ -328,6 +329,7 @@ def _knn_forward(coords: torch.Tensor, D: int, row_splits, K: int, direction, n_
             s = stats.tolist()
             with _STATS_LOCK:
                 last_stats.update(distance_evaluations=s[0], candidate_chunks=s[1], pool_prunes=s[2],
+                                  matrix_search_handed_over=s[3], matrix_search_collected=s[5],
                                   n_bins=nb, n_vert=n, K=K, n_coords=D)
     if nbr_sorted is None:
         nbr_sorted = torch.empty((0, K), dtype=torch.int32, device=dev)

@@ -26,7 +26,9 @@ tile_aggregation_backward = True
 # The neighbour set, the distances and the gradients are the same either way.
 sorted_neighbours = False
 
-# Searches over points with 5 to 8 coordinates (K <= 256) screen their candidates on the matrix cores and compute exact
-# distances only for the pairs that can still matter.  False: the vector-unit search, as for every other shape.  Same
-# neighbours and bit-identical distances either way.
+# Searches over points with 5 to 8 coordinates (K <= 256, events of at most 65535 points) can screen their candidates
+# on the matrix cores and compute exact distances only for the pairs that can still matter.  True: the library decides
+# by the event sizes (where bounding boxes thin the candidates out well the vector-unit search is faster); False:
+# always the vector-unit search; "always": the matrix cores wherever that search can run.  Same neighbours and
+# bit-identical distances either way.
 matrix_search = True

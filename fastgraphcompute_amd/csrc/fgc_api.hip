@@ -1,6 +1,7 @@
 // Whole-call entry points and bookkeeping of libfgc_hip.so.
 #include "fgc_common.h"
 #include "fgc_internal.h"
+#include <algorithm>
 #include <cstdlib>
 #include <mutex>
 
@@ -24,7 +25,7 @@ extern "C" const char *fgc_error_string(int code)
 
 namespace {
 struct KnnWorkspace {
-    size_t geom, partial, keys, vals, sort, sort_alt_vals, bb, sc, sp, redo, sdir, box_lo, box_hi, sbox_lo, sbox_hi, total;
+    size_t geom, partial, keys, vals, sort, sort_alt_vals, bb, sc, sp, spa, grp, mfstat, redo, sdir, box_lo, box_hi, sbox_lo, sbox_hi, total;
     bool with_sp;
     int ldc;
 };
@@ -58,6 +59,9 @@ KnnWorkspace plan(int64_t n, int D, int K, int nbd, const int64_t *n_bins, int n
     w.sc = take((size_t)w.ldc * D * 4);
     w.with_sp = fgc_knn_uses_mfma(D, K);     // rows of 8 floats for the matrix-core search
     w.sp = take(w.with_sp ? (size_t)w.ldc * 32 : 0);
+    w.spa = take(w.with_sp ? (size_t)w.ldc * 32 : 0);    // float16 operands of the same points
+    w.grp = take(w.with_sp ? (size_t)((w.ldc / 64 + FGC_MF_GROUP_CHUNKS - 1) / FGC_MF_GROUP_CHUNKS) * FGC_MF_GRP_FLOATS * 4 : 0);
+    w.mfstat = take(w.with_sp ? 8 : 0);
     w.redo = take(w.with_sp ? (size_t)w.ldc : 0);   // flags of the queries the matrix-core search leaves to the vector search
     w.sdir = take(with_dir ? (size_t)n : 0);
     w.box_lo = take((size_t)(w.ldc / 64) * D * 4);
@@ -185,8 +189,12 @@ extern "C" int fgc_binned_knn_prepare_ld_f32(const float *d_coords, int64_t n_ve
     rc = fgc_launch_gather_sorted(d_coords, ld_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir,
                                   w.with_sp ? (float *)(ws + w.sp) : nullptr, fgc_knn_sp_half(n_coords), s);
     if (rc) return rc;
-    return fgc_launch_chunk_boxes(sc, (int)n_vert, n_coords, w.ldc, (float *)(ws + w.box_lo),
-                                  (float *)(ws + w.box_hi), (float *)(ws + w.sbox_lo), (float *)(ws + w.sbox_hi), s);
+    rc = fgc_launch_chunk_boxes(sc, (int)n_vert, n_coords, w.ldc, (float *)(ws + w.box_lo),
+                                (float *)(ws + w.box_hi), (float *)(ws + w.sbox_lo), (float *)(ws + w.sbox_hi), s);
+    if (rc || !w.with_sp) return rc;
+    return fgc_launch_mf_operands((const float *)(ws + w.sp), (const float *)(ws + w.box_lo),
+                                  (const float *)(ws + w.box_hi), (int)n_vert, n_coords, w.ldc, (float *)(ws + w.grp),
+                                  ws + w.spa, (unsigned *)(ws + w.mfstat), s);
 }
 
 namespace {
@@ -220,10 +228,31 @@ int knn_search(float tau0, int32_t *d_nbr_sorted, int64_t n_vert, int32_t n_coor
     a.out_sorted = d_nbr_sorted;
     a.out_idx = d_idx; a.out_dist = d_distsq; a.stats = (unsigned long long *)d_stats;
     a.sp = c.w.with_sp ? (const float *)(ws + c.w.sp) : nullptr;
+    a.spa = c.w.with_sp ? (const void *)(ws + c.w.spa) : nullptr;
+    a.grp = c.w.with_sp ? (const float *)(ws + c.w.grp) : nullptr;
+    a.mfstat = c.w.with_sp ? (const unsigned *)(ws + c.w.mfstat) : nullptr;
     a.redo = nullptr;
     // many coordinates: candidates screened on the matrix cores (a radius bound keeps the vector search, which
     // culls by it from the first bin row on)
-    if (a.sp && !(tf_compat & FGC_KNN_NO_MATRIX) && !(tau0 < INFINITY)) {
+    // Many coordinates and events that the bounding boxes cannot thin out: the matrix-core search.  Measured on
+    // uniform and clustered points with 1 000 to 65 000 points per event: it wins up to about 1024 * 4^(D - 5)
+    // points per event (twice that from K = 64 on), where the size is the one a typical point sees, sum n_e^2 / n.
+    // It stores candidates as 16-bit positions inside their event, so no event may exceed 65535 points.
+    int64_t largest_event = 0;
+    double sum_sq = 0;
+    for (int r = 1; r < n_rs; r++) {
+        const int64_t ne = row_splits_host[r] - row_splits_host[r - 1];
+        largest_event = std::max(largest_event, ne);
+        sum_sq += (double)ne * (double)ne;
+    }
+    const double typical_event = n_vert > 0 ? sum_sq / (double)n_vert : 0.0;
+    double limit = 1024.0;
+    for (int d = 5; d < n_coords; d++) limit *= 4.0;
+    if (K >= 64) limit *= 2.0;
+    limit = std::min(limit, 32768.0);
+    const bool force = (tf_compat & FGC_KNN_FORCE_MATRIX) != 0;
+    if (a.sp && !(tf_compat & FGC_KNN_NO_MATRIX) && !(tau0 < INFINITY) && largest_event <= 65535 &&
+        (typical_event <= limit || force)) {
         a.redo = (unsigned char *)(ws + c.w.redo);
         return a.stats ? fgc_launch_knn_mfma_stats(a, (hipStream_t)stream) : fgc_launch_knn_mfma(a, (hipStream_t)stream);
     }

@@ -20,6 +20,9 @@ struct KnnArgs {
     const float *sc;            // sorted coordinates, structure of arrays [D][ldc]
     int ldc;
     const float *sp;            // sorted coordinates as rows of 8 floats (matrix-core search only), or NULL
+    const void *spa;            // the same points as float16 matrix operands relative to their group's centre, and
+    const float *grp;           // the group records (fgc_launch_mf_operands); matrix-core search only
+    const unsigned *mfstat;     // [2] chunks counted / chunks of groups far wider than the chunk (fgc_launch_mf_operands)
     const uint32_t *skeys;      // sorted key per point: (flat bin << key_shift) | Hilbert index inside the bin
     int key_shift;
     const float *box_lo;        // per 64-point chunk bounding boxes [D][n_chunks]
@@ -55,5 +58,16 @@ int fgc_launch_knn_stats(const KnnArgs &a, hipStream_t s);  // the same search, 
 // needs a.sp.  Same rows as fgc_launch_knn up to the order inside a row and the choice between exactly tied candidates.
 bool fgc_knn_uses_mfma(int D, int K);
 inline int fgc_knn_sp_half(int D) { return D <= 6 ? 3 : 4; }   // coordinates per half row of sp
+// Float16 operands of the matrix-core search.  A group is 16 consecutive chunks (1024 sorted points); grp[g] holds 16
+// floats: the centre of the group's bounding box in the layout of sp (8), the scale sigma_g (a power of two with
+// |c - centre| sigma_g <= 150 for every point of the group), the squared radius R_g^2 of the box, padding.  spa holds
+// per point two halves of 8 float16: (c - centre) sigma_g for the half's coordinates (4, zero padded), then in the
+// first half |c - centre|^2 sigma_g^2 (1 - 1.03 * 2^-10) as a (high, low) pair and 1, 1 - zeros in the second half.  A
+// point with a non-finite coordinate, and the padding rows, carry an infinite norm.  mfstat[0] counts the chunks,
+// mfstat[1] those whose group's squared radius is more than 24 times the chunk's own.
+#define FGC_MF_GROUP_CHUNKS 16
+#define FGC_MF_GRP_FLOATS 16
+int fgc_launch_mf_operands(const float *sp, const float *box_lo, const float *box_hi, int n, int D, int ldc,
+                           float *grp, void *spa, unsigned *mfstat, hipStream_t s);
 int fgc_launch_knn_mfma(const KnnArgs &a, hipStream_t s);
 int fgc_launch_knn_mfma_stats(const KnnArgs &a, hipStream_t s);

@@ -70,27 +70,120 @@ __device__ __forceinline__ float mf_wave_max_f(float v) { return -mf_wave_min_f(
 // value of the partner lane (lane ^ 32)
 __device__ __forceinline__ int mf_other_half(int v) { return fgc_xor_lane<32>(v); }
 
-// a bound x on the float16 screening value s, widened so that it bounds the exact squared distance d^2 of every pair
-// whose s is below x: s >= d^2 - 2^-9 * 1.03 (|q'|^2 + |c'|^2) and |c'|^2 <= 2 |q'|^2 + 2 d^2 give
-// d^2 <= (s + 3 * 2^-9 * 1.03 |q'|^2) / (1 - 2^-8 * 1.03)
-__device__ __forceinline__ float mf_widen(float x, float qn) { return (x + qn * 0x1p-7f) * (1.0f + 0x1.1p-8f) + 1e-30f; }
 
 using MfMax = std::integral_constant<int, 0>;
 using MfHist = std::integral_constant<int, 1>;
 using MfCollect = std::integral_constant<int, 2>;
 
+constexpr float MF_SHRINK16 = 1.0f - 0x1.08p-10f;    // 1 - 1.03 * 2^-10
+
+// Float16 operands of the candidates (see fgc_internal.h): one wavefront per chunk, lane = point.
+__global__ __launch_bounds__(256) void k_mf_operands(const float4 *__restrict__ sp4, const float *__restrict__ box_lo,
+                                                     const float *__restrict__ box_hi, int n, int D, int DH, int ldc,
+                                                     int n_chunks, float *__restrict__ grp, uint4 *__restrict__ spa,
+                                                     unsigned *__restrict__ mfstat)
+{
+    const int lane = fgc_lane();
+    const int c = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
+    if (c >= n_chunks) return;
+    const int g = c / FGC_MF_GROUP_CHUNKS;
+    // bounding box of the group, coordinate d in lane d
+    float lo = INFINITY, hi = -INFINITY;
+    if (lane < D)
+        for (int cc = g * FGC_MF_GROUP_CHUNKS; cc < min((g + 1) * FGC_MF_GROUP_CHUNKS, n_chunks); cc++) {
+            lo = fminf(lo, box_lo[(size_t)lane * n_chunks + cc]);
+            hi = fmaxf(hi, box_hi[(size_t)lane * n_chunks + cc]);
+        }
+    // How wide is the group against its own chunks?  Where a group of 1024 points spans several clusters while its
+    // chunks of 64 sit inside one, the float16 screening error (proportional to the group's squared radius) exceeds
+    // the neighbour distances and the matrix-core search could only hand its queries on: counted here, decided there.
+    {
+        const float clo = lane < D ? box_lo[(size_t)lane * n_chunks + c] : 0.f;
+        const float chi = lane < D ? box_hi[(size_t)lane * n_chunks + c] : 0.f;
+        const float ch = (lane < D && fabsf(clo) < INFINITY && fabsf(chi) < INFINITY && chi >= clo) ? 0.5f * chi - 0.5f * clo : 0.f;
+        const float gh = (lane < D && fabsf(lo) < INFINITY && fabsf(hi) < INFINITY && hi >= lo) ? 0.5f * hi - 0.5f * lo : 0.f;
+        const float rc2 = fgc_wave_sum(ch * ch), rg2 = fgc_wave_sum(gh * gh);
+        if (lane == 0 && c * 64 < n) {
+            atomicAdd(&mfstat[0], 1u);
+            if (rg2 > 24.f * rc2) atomicAdd(&mfstat[1], 1u);
+        }
+    }
+    float ctr = 0.5f * lo + 0.5f * hi, half = 0.5f * hi - 0.5f * lo;
+    if (lane >= D) { ctr = 0.f; half = 0.f; }
+    else if (!(fabsf(lo) < INFINITY && fabsf(hi) < INFINITY)) { ctr = 0.f; half = lo > hi ? 0.f : INFINITY; }   // lo > hi: no finite point
+    const float R2 = fgc_wave_sum(half * half) * (1.0f + 0x1p-20f);
+    // sigma: the power of two with 75 < R sigma <= 150
+    float sigma;
+    if (!(R2 < INFINITY)) sigma = 0x1p-40f;
+    else if (!(R2 > 0.f)) sigma = 0x1p40f;
+    else {
+        const float want = 150.f / sqrtf(R2);
+        sigma = __uint_as_float(min(max(__float_as_uint(want) & 0xff800000u, 0x20000000u), 0x5f000000u));
+    }
+    // the centre in the layout of sp: float f of a row is coordinate f (f < 4) or DH + f - 4
+    float cf[8];
+#pragma unroll
+    for (int f = 0; f < 8; f++) {
+        const int d = f < 4 ? f : DH + f - 4;
+        const bool used = (f < 4 ? f < DH : true) && d < D;
+        cf[f] = used ? fgc_readlane_f(ctr, d < 63 ? d : 63) : 0.f;
+    }
+    if (lane == 0 && c % FGC_MF_GROUP_CHUNKS == 0) {
+        float *rec = grp + (size_t)g * FGC_MF_GRP_FLOATS;
+#pragma unroll
+        for (int f = 0; f < 8; f++) rec[f] = cf[f];
+        rec[8] = sigma; rec[9] = R2;
+#pragma unroll
+        for (int f = 10; f < FGC_MF_GRP_FLOATS; f++) rec[f] = 0.f;
+    }
+    const int i = c * 64 + lane;
+    const float4 x0 = sp4[(size_t)i * 2], x1 = sp4[(size_t)i * 2 + 1];
+    const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+    float r[8], rn = 0.f;
+#pragma unroll
+    for (int f = 0; f < 8; f++) {
+        r[f] = __builtin_fmaf(x[f], sigma, -cf[f] * sigma);
+        rn = __builtin_fmaf(r[f], r[f], rn);
+    }
+    const bool ok = i < n && rn < 60000.f;
+    const float rne = rn * MF_SHRINK16;
+    const _Float16 nh = (_Float16)rne;
+    const _Float16 nl = (_Float16)(rne - (float)nh);
+    union { fgc_h8 h; uint4 u; } a0, a1;
+    const _Float16 zero = (_Float16)0.f, one = (_Float16)1.f, inf = (_Float16)INFINITY;
+    a0.h = fgc_h8{ok ? (_Float16)r[0] : zero, ok ? (_Float16)r[1] : zero, ok ? (_Float16)r[2] : zero,
+                  ok ? (_Float16)r[3] : zero, ok ? nh : inf, ok ? nl : zero, one, one};
+    a1.h = fgc_h8{ok ? (_Float16)r[4] : zero, ok ? (_Float16)r[5] : zero, ok ? (_Float16)r[6] : zero,
+                  ok ? (_Float16)r[7] : zero, zero, zero, zero, zero};
+    spa[(size_t)i * 2] = a0.u;
+    spa[(size_t)i * 2 + 1] = a1.u;
+}
+
+int fgc_launch_mf_operands(const float *sp, const float *box_lo, const float *box_hi, int n, int D, int ldc, float *grp,
+                           void *spa, unsigned *mfstat, hipStream_t s)
+{
+    const int n_chunks = ldc / 64;
+    int rc = fgc_fill_u32(mfstat, 0u, 2, s);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_mf_operands, dim3((unsigned)fgc_cdiv(n_chunks, 4)), dim3(256), 0, s, (const float4 *)sp, box_lo,
+                       box_hi, n, D, fgc_knn_sp_half(D), ldc, n_chunks, grp, (uint4 *)spa, mfstat);
+    FGC_LAUNCH_CHECK();
+    return FGC_OK;
+}
+
 // D: coordinates per point, padded to an even number (6 or 8; a padding coordinate is 0 for every point and adds an
 // exact +0 to every distance).  NSEG: ceil(K / 64).  PS: ceil(column height / 64).
 template <int D, int NSEG, int PS, bool STATS>
-__global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
+__global__ __launch_bounds__(64, 4) void k_knn_mf(KnnArgs a)
 {
     constexpr int DH = D / 2;             // coordinates per half of the wavefront
     extern __shared__ unsigned s_mf[];
     const int CAP = a.pool_cap;           // column height: histogram buckets = collected candidates per query at most
-    unsigned *col = s_mf;                 // [CAP][32]: per query (column) histogram counts, later collected sorted
-                                          // positions.  Word (b, q) lies in bank q or q + 32: accesses with lane =
-                                          // query never collide between queries, whatever rows they touch
-    uint2 *rowbuf = (uint2 *)(s_mf + 32 * CAP);   // [NSEG * 64] one query's selected (distance, position) pairs
+    unsigned short *col = (unsigned short *)s_mf;   // [CAP][32] 16-bit entries: per query (column) histogram counts,
+                                          // later the collected candidates as positions inside their event - which is why
+                                          // this kernel takes events of at most 65535 points.  Half the bytes of 32-bit
+                                          // entries: four wavefronts per SIMD instead of two
+    uint2 *rowbuf = (uint2 *)(s_mf + 16 * CAP);   // [NSEG * 64] one query's selected (distance, position) pairs
 
     const int lane = fgc_lane();
     const int q = lane & 31, h = lane >> 5;
@@ -99,6 +192,11 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
     const int nq = min(MF_QT, a.n - qbeg);
     const bool isq = q < nq;
     const int qs = qbeg + (isq ? q : 0);
+    // strongly clustered points (counted by the preparation stage): everything goes to the vector search
+    if (a.mfstat[1] * 4u > a.mfstat[0]) {
+        if (h == 0 && isq) a.redo[qs] = 1;
+        return;
+    }
     const int K = a.K;
     const int Dn = a.D;                   // coordinates the points really have (D or D - 1)
     const float4 *__restrict__ sp4 = (const float4 *)a.sp;   // [ldc][2]: coordinates h * DH .. h * DH + DH - 1 in half h
@@ -152,13 +250,24 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
     int n_own = 0;           // collected candidates of this lane: lane (0, q) fills column q from the top, (1, q) from the bottom
     bool over = false;       // the query is left to the vector search (column full, or out of the float16 range)
     const float NBm1 = (float)(CAP - 1);
-    // float16 screening (wave-uniform scale, per-lane operands)
-    float sig = 1.f;         // sigma: power of two
-    float osig[DH];          // o * sigma
-    float thr = -INFINITY;   // collect pass: candidates with accumulator below this are taken (units: sigma^2)
-    float hsc = 0.f;         // histogram pass: the accumulators hold s * sigma^2 * hsc, hsc a power of two; bucket = trunc
-    fgc_h8 bh = {0, 0, 0, 0, 0, 0, 0, 0};   // B operand: (-2 q' sigma S) x 4, then for h = 0: S, S, |q'|^2 sigma^2 S (1 - m) as (high, low)
-    constexpr float SHRINK16 = 1.0f - 0x1.08p-10f;
+    // float16 screening: the candidates' operands are relative to the centre of their group of 8 chunks, the query's
+    // operand is recomputed whenever the scan enters another group
+    const uint4 *__restrict__ spa4 = (const uint4 *)a.spa;
+    float qh4[4];            // the query's coordinates of this lane's half
+    {
+        const float4 qm = sp4[(size_t)qs * 2 + h];
+        qh4[0] = qm.x; qh4[1] = qm.y; qh4[2] = qm.z; qh4[3] = qm.w;
+    }
+    int cur_g = -1;          // group the B operand stands for
+    int pg_id = -1;          // group whose record sits in pg_c / pg_s
+    float4 pg_c = make_float4(0.f, 0.f, 0.f, 0.f);
+    float2 pg_s = make_float2(1.f, 0.f);
+    const int n_groups = (a.n_chunks + FGC_MF_GROUP_CHUNKS - 1) / FGC_MF_GROUP_CHUNKS;
+    float hsc = 0.f;         // histogram pass: bucket = trunc(s * hsc), hsc a power of two (0: the query takes no part)
+    float thr = -INFINITY;   // collect pass: candidates with accumulator below this are taken (units: sigma_g^2)
+    int ev_base = 0;         // first sorted position of the query's event: collected candidates are stored relative to it
+    bool collecting = false; // collect pass (accumulators in units of sigma_g^2) or histogram pass (units of 1 / hsc)
+    fgc_h8 bh = {0, 0, 0, 0, 0, 0, 0, 0};   // B operand: (-2 q_g sigma S) x 4, then for h = 0: S, S, |q_g|^2 sigma^2 S (1 - m) as (high, low)
 
     unsigned long long nev = 0;
     unsigned nchunks = 0, n_range = 0, n_over = 0, n_coll = 0;
@@ -169,6 +278,10 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
         if (a.sdir && valid) { const unsigned char dd = a.sdir[jc]; if (dd == 1 || dd == 2) valid = false; }
         return valid;
     };
+
+    // The float16 screening value s of a pair is at most 2^-9 * 1.02 (|q_g|^2 + |r|^2) below its squared distance
+    // d^2 (q_g, r: query and candidate relative to the centre of the candidate's group); with |q_g| <= d + |r| and
+    // |r|^2 <= R_g^2 that gives d^2 <= (s + 3 * 2^-9 * 1.02 R_g^2) / (1 - 2^-8 * 1.02).
 
     // ---- one tile in float32 (step A): the accumulators hold s ----
     auto tile_f32 = [&](int jt, const float4 cc, int ev_j0, int ev_j1, int &nok) -> fgc_f32x16 {
@@ -190,52 +303,78 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
         if (STATS) nev += (unsigned long long)nok * (unsigned)__popcll(fgc_ballot(ing && h == 0));
         return acc;
     };
-    // ---- one tile in float16: the accumulators hold s sigma^2 S (S = 1 in the collect pass) ----
-    auto tile_f16 = [&](int jt, const float4 cc, int ev_j0, int ev_j1, int &nok) -> fgc_f32x16 {
-        const bool valid = usable(jt + q, ev_j0, ev_j1);
-        const float ct[4] = {cc.x, cc.y, cc.z, cc.w};
-        float t[4] = {0.f, 0.f, 0.f, 0.f};
+    // ---- one tile in float16: the accumulators hold s sigma_g^2 S.  `inside`: every candidate of the tile belongs
+    //      to the event and no direction flags are in use (nothing to mask) ----
+    auto tile_f16 = [&](int jt, uint4 av, bool inside, int ev_j0, int ev_j1) -> fgc_f32x16 {
+        if (!inside) {
+            // an unusable candidate gets an infinite norm (element 4 of the first half)
+            if (!usable(jt + q, ev_j0, ev_j1) && h == 0) av.z = 0x00007c00u;
+        }
+        union { uint4 u; fgc_h8 v; } cv;
+        cv.u = av;
+        fgc_f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(cv.v, bh, acc, 0, 0, 0);
+        if (STATS) nev += 32ull * (unsigned)__popcll(fgc_ballot(ing && h == 0));
+        return acc;
+    };
+    // B operand of the float16 tiles for group g.  S is chosen so that the accumulators come out in the units of the
+    // pass: sigma_g^2 S = hsc in a histogram pass, S = 1 in the collect pass (thr follows sigma_g).  A query whose
+    // operands leave the float16 range gets an infinite accumulator if the group is farther away than its bound,
+    // and is given up otherwise.
+    auto set_group = [&](int g) {
+        cur_g = g;
+        // the record of the group: from the registers filled ahead of time when the scan moved on as expected
+        if (g != pg_id) {
+            const float *rec = a.grp + (size_t)g * FGC_MF_GRP_FLOATS;
+            pg_c = *(const float4 *)(rec + 4 * h);
+            pg_s = *(const float2 *)(rec + 8);
+        }
+        const float4 gc = pg_c;
+        const float sg = pg_s.x, R2 = pg_s.y;
+        {
+            // ask for the next group's record now
+            pg_id = min(g + 1, n_groups - 1);
+            const float *rec = a.grp + (size_t)pg_id * FGC_MF_GRP_FLOATS;
+            pg_c = *(const float4 *)(rec + 4 * h);
+            pg_s = *(const float2 *)(rec + 8);
+        }
+        const float gcf[4] = {gc.x, gc.y, gc.z, gc.w};
+        float qg[4] = {0.f, 0.f, 0.f, 0.f};
         float part = 0.f;
 #pragma unroll
         for (int j = 0; j < DH; j++) {
-            t[j] = __builtin_fmaf(ct[j], sig, -osig[j]);     // (c - o) sigma, rounded once
-            part = __builtin_fmaf(t[j], t[j], part);
+            qg[j] = qh4[j] - gcf[j];
+            part = __builtin_fmaf(qg[j], qg[j], part);
         }
-        const float cn = fgc_halve_pair<32>(part, part, lane);
-        const bool ok = valid && cn < 60000.f;       // beyond the float16 range: farther than anything that matters
-        const float cne = cn * SHRINK16;
-        const _Float16 ch = (_Float16)cne;
-        const _Float16 cl = (_Float16)(cne - (float)ch);
-        const fgc_f2 p0 = {ok ? t[0] : 0.f, ok ? t[1] : 0.f}, p1 = {ok ? t[2] : 0.f, ok ? t[3] : 0.f};
-        const fgc_h2 h0 = __builtin_convertvector(p0, fgc_h2), h1 = __builtin_convertvector(p1, fgc_h2);
-        const _Float16 zero = (_Float16)0.f, one = (_Float16)1.f, inf = (_Float16)INFINITY;
-        const fgc_h8 ah = {h0[0], h0[1], h1[0], h1[1], h ? zero : (ok ? ch : inf), h ? zero : (ok ? cl : zero),
-                           h ? zero : one, h ? zero : one};
-        fgc_f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh, acc, 0, 0, 0);
-        nok = __popcll(fgc_ballot(ok && h == 0));
-        if (STATS) nev += (unsigned long long)nok * (unsigned)__popcll(fgc_ballot(ing && h == 0));
-        return acc;
-    };
-    // B operand of the float16 tiles for the scale S (a power of two); a query whose operands leave the float16 range
-    // (its bound is tiny against the spread of the wavefront's queries: nothing could be screened anyway) is given up
-    auto set_b16 = [&](float S) {
-        const float f = -2.f * sig * S;
-        float t[4] = {0.f, 0.f, 0.f, 0.f};
+        const float qgn = fgc_halve_pair<32>(part, part, lane);
+        const float S = collecting ? 1.f : hsc / (sg * sg);          // powers of two (0 for a query that takes no part)
+        const float f = -2.f * sg * S;
+        float t[4];
 #pragma unroll
-        for (int j = 0; j < DH; j++) t[j] = tq[j] * f;
-        const float qs2 = qn * sig * sig * S * SHRINK16;
-        const bool fits = ing && S < 30000.f && qs2 < 60000.f && fabsf(t[0]) < 60000.f && fabsf(t[1]) < 60000.f &&
-                          fabsf(t[2]) < 60000.f && fabsf(t[3]) < 60000.f;
-        if (ing && !fits) { over = true; if (STATS) n_range++; }
-        const _Float16 qh = (_Float16)qs2;
-        const _Float16 ql = (_Float16)(qs2 - (float)qh);
-        const _Float16 zero = (_Float16)0.f, Sh = (_Float16)S;
-        const bool on = fits && !over;
+        for (int j = 0; j < 4; j++) t[j] = qg[j] * f;
+        // histogram pass: the group's share of the screening error goes on top, so that the histogram counts upper
+        // bounds of the squared distances, s + 3 * 2^-9 * 1.02 R_g^2 (times 1 / (1 - 2^-8 * 1.02), applied at the cut):
+        // a wide group far away only blurs its own candidates
+        const float qs2 = (qgn * MF_SHRINK16 + (collecting ? 0.f : R2 * 0x1p-7f)) * (sg * sg) * S;
+        const bool part_of = ing && !over && (collecting || hsc > 0.f);
+        bool fits = S < 30000.f && qs2 < 60000.f && fabsf(t[0]) < 60000.f && fabsf(t[1]) < 60000.f &&
+                    fabsf(t[2]) < 60000.f && fabsf(t[3]) < 60000.f;
+        fits = fits && (fgc_ballot(fits) >> (lane ^ 32) & 1ull);    // both lanes of the query
+        // the whole group beyond the query's bound?  (|q_g| - R_g)^2 > bound
+        const float gapr = __builtin_amdgcn_sqrtf(qgn) * (1.0f - 0x1p-20f) - __builtin_amdgcn_sqrtf(R2) * (1.0f + 0x1p-20f);
+        const bool beyond = gapr > 0.f && gapr * gapr > bound * (1.0f + 0x1p-10f);
+        if (part_of && !fits && !beyond) { over = true; if (STATS) n_range++; }
+        const bool on = part_of && fits && !over;
+        const bool far = part_of && !fits && beyond;
+        const _Float16 zero = (_Float16)0.f, inf = (_Float16)INFINITY;
+        const _Float16 Sh = on ? (_Float16)S : (far ? (_Float16)1.f : zero);
+        const _Float16 qh = on ? (_Float16)qs2 : (far ? inf : zero);
+        const _Float16 ql = on ? (_Float16)(qs2 - (float)qh) : zero;
         bh[0] = on ? (_Float16)t[0] : zero; bh[1] = on ? (_Float16)t[1] : zero;
         bh[2] = on ? (_Float16)t[2] : zero; bh[3] = on ? (_Float16)t[3] : zero;
-        bh[4] = (on && !h) ? Sh : zero; bh[5] = (on && !h) ? Sh : zero;
-        bh[6] = (on && !h) ? qh : zero; bh[7] = (on && !h) ? ql : zero;
+        bh[4] = h ? zero : Sh; bh[5] = h ? zero : Sh;
+        bh[6] = h ? zero : qh; bh[7] = h ? zero : ql;
+        if (collecting) thr = on ? bound * (sg * sg) * (1.0f + 0x1p-20f) : -INFINITY;
     };
 
     // accumulator v of lane (h, q): candidate row 8 (v / 4) + 4 h + v % 4, query q
@@ -244,23 +383,25 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
 #pragma unroll
             for (int v = 0; v < 16; v++) mx = (acc[v] < INFINITY) ? fmaxf(mx, acc[v]) : mx;
         } else if constexpr (decltype(mode)::value == 1) {
-            unsigned *mycol = col + q;
+            // two columns share a 32-bit word: the count of query q is its half (q & 1); no count passes 65535
+            unsigned *mycol = s_mf + (q >> 1);
+            const unsigned inc = (q & 1) ? 0x10000u : 1u;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int b = (int)__builtin_amdgcn_fmed3f(acc[v], 0.f, NBm1);
-                atomicAdd(mycol + (b << 5), 1u);
+                atomicAdd(mycol + (b << 4), inc);
             }
         } else {
             // the two lanes of a query share what is left of its column evenly for this tile; a candidate that
             // finds no room leaves the query to the vector search
             const int tot = n_own + mf_other_half(n_own);
             const int lim = n_own + ((CAP - tot) >> 1);
-            const int jh = jt + 4 * h;
+            const int jh = jt + 4 * h - ev_base;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 if (acc[v] < thr) {
                     if (n_own < lim) {
-                        col[((h ? CAP - 1 - n_own : n_own) << 5) + q] = (unsigned)(jh + 8 * (v / 4) + (v % 4));
+                        col[((h ? CAP - 1 - n_own : n_own) << 5) + q] = (unsigned short)(jh + 8 * (v / 4) + (v % 4));
                         n_own++;
                     } else over = true;
                 }
@@ -268,32 +409,48 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
         }
     };
 
-    // both tiles of chunk c; the coordinates were requested by prefetch(c), those of chunk c_next (if >= 0) are
+    // both tiles of chunk c; the operands were requested by prefetch(c), those of chunk c_next (if >= 0) are
     // requested here, before the matrix products of this chunk are worked through
     float4 pre0, pre1;
-    auto prefetch = [&](int c) {
+    uint4 prh0, prh1;
+    auto prefetch32 = [&](int c) {
         const int j = c << 6;
         pre0 = sp4[(size_t)(j + q) * 2 + h];
         pre1 = sp4[(size_t)(j + 32 + q) * 2 + h];
     };
-    auto chunk = [&](auto mode, int c, int c_next, int ev_j0, int ev_j1) -> int {
+    const unsigned lane_off = (unsigned)(q * 2 + h) * 16u;       // this lane's operand inside a tile of 32 x 32 bytes
+    auto prefetch = [&](int c) {
+        const char *base = (const char *)spa4 + (size_t)c * 2048;  // wave-uniform base + 32-bit lane offset
+        prh0 = *(const uint4 *)(base + lane_off);
+        prh1 = *(const uint4 *)(base + 1024 + lane_off);
+    };
+    auto chunk32 = [&](int c, int ev_j0, int ev_j1) -> int {
         const int j = c << 6;
-        const float4 c0 = pre0, c1 = pre1;
-        if (c_next >= 0) prefetch(c_next);
+        prefetch32(c);
         if (STATS) nchunks++;
         int nok0 = 0, nok1 = 0;
         const bool two = j + 32 < ev_j1;
-        fgc_f32x16 acc0, acc1;
-        if constexpr (decltype(mode)::value == 0) {
-            acc0 = tile_f32(j, c0, ev_j0, ev_j1, nok0);
-            if (two) acc1 = tile_f32(j + 32, c1, ev_j0, ev_j1, nok1);
-        } else {
-            acc0 = tile_f16(j, c0, ev_j0, ev_j1, nok0);
-            if (two) acc1 = tile_f16(j + 32, c1, ev_j0, ev_j1, nok1);
+        const fgc_f32x16 acc0 = tile_f32(j, pre0, ev_j0, ev_j1, nok0);
+        tile_post(MfMax{}, j, acc0);
+        if (two) {
+            const fgc_f32x16 acc1 = tile_f32(j + 32, pre1, ev_j0, ev_j1, nok1);
+            tile_post(MfMax{}, j + 32, acc1);
         }
+        return nok0 + nok1;
+    };
+    auto chunk = [&](auto mode, int c, int c_next, int ev_j0, int ev_j1) {
+        const int j = c << 6;
+        const uint4 c0 = prh0, c1 = prh1;
+        if (c_next >= 0) prefetch(c_next);
+        if (STATS) nchunks++;
+        if ((c / FGC_MF_GROUP_CHUNKS) != cur_g) set_group(c / FGC_MF_GROUP_CHUNKS);
+        const bool inside = !a.sdir && j >= ev_j0 && j + 64 <= ev_j1;
+        const bool two = j + 32 < ev_j1;
+        const fgc_f32x16 acc0 = tile_f16(j, c0, inside, ev_j0, ev_j1);
+        fgc_f32x16 acc1;
+        if (two) acc1 = tile_f16(j + 32, c1, inside, ev_j0, ev_j1);
         tile_post(mode, j, acc0);
         if (two) tile_post(mode, j + 32, acc1);
-        return nok0 + nok1;
     };
     // a chunk of an event that is collected whole: every usable candidate goes to every query of the event
     auto chunk_all = [&](int c, int ev_j0, int ev_j1) {
@@ -307,7 +464,7 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
                 const int r = 8 * (v / 4) + 4 * h + (v % 4);
                 if (ing && ((um >> r) & 1u)) {
                     if (n_own < lim) {
-                        col[((h ? CAP - 1 - n_own : n_own) << 5) + q] = (unsigned)(jt + r);
+                        col[((h ? CAP - 1 - n_own : n_own) << 5) + q] = (unsigned short)(jt + r - ev_base);
                         n_own++;
                     } else over = true;
                 }
@@ -316,21 +473,20 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
     };
 
     auto zero_columns = [&]() {
-        for (int i = lane; i < 32 * CAP; i += 64) col[i] = 0u;
+        for (int i = lane; i < 16 * CAP; i += 64) s_mf[i] = 0u;
     };
 
-    // histogram scale: the largest power of two S with bound sigma^2 S <= CAP - 2, so that the range [0, bound) falls
+    // histogram scale: the largest power of two with bound * hsc <= CAP - 2, so that the range [0, bound) falls
     // on the buckets 0 .. CAP - 2 (the last bucket takes everything beyond)
     auto set_hist_scale = [&]() {
         hsc = 0.f;
         if (ing && bound < INFINITY && bound > 0.f && !over) {
-            const float want = (NBm1 - 1.f) / (bound * sig * sig);
-            if (want < INFINITY && want > 1e-30f)
+            const float want = (NBm1 - 1.f) / bound;
+            if (want < 0x1p100f && want > 0x1p-100f)
                 hsc = __uint_as_float(__float_as_uint(want) & 0xff800000u);     // mantissa cleared: rounded down to 2^e
         }
-        set_b16(hsc > 0.f ? hsc : 1.f);
-        if (!(hsc > 0.f)) bh = fgc_h8{0, 0, 0, 0, 0, 0, 0, 0};
-        if (over) hsc = 0.f;
+        collecting = false;
+        cur_g = -1;
     };
     // bucket where the running count of the query's histogram reaches K -> bound on the K-th smallest squared distance:
     // the upper edge of that bucket, widened by the screening error (unchanged when fewer than K candidates lie
@@ -341,10 +497,8 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
             cum += (int)col[(b << 5) + q];
             if (cum >= K && bstar == CAP - 1) bstar = b;
         }
-        if (ing && bstar < CAP - 1 && hsc > 0.f) {
-            const float edge = (float)(bstar + 1) / (hsc * sig * sig);
-            bound = fminf(bound, mf_widen(edge, qn));
-        }
+        if (ing && bstar < CAP - 1 && hsc > 0.f && !over)
+            bound = fminf(bound, (float)(bstar + 1) / hsc * (1.0f + 0x1.1p-8f) + 1e-30f);
     };
 
     // pass over the event's chunks outside [skip_lo, skip_hi] that the queries' balls of squared radius `reach`
@@ -408,6 +562,11 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
             todo &= ~gm;
             ing = (gm >> lane) & 1ull;
             const int ev_j0 = bb[gev * bpe], ev_j1 = bb[(gev + 1) * bpe];
+            if (ing) ev_base = ev_j0;
+            if (ev_j1 - ev_j0 > 65535) {               // positions inside the event must fit 16 bits
+                if (ing) over = true;
+                continue;
+            }
             const int c_lo = ev_j0 >> 6, c_hi = (ev_j1 - 1) >> 6;
             const int own = qbeg >> 6;
             const int seed_w = (K + MF_SEED_K - 1) / MF_SEED_K;
@@ -421,8 +580,7 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
                 for (int k = 0; k <= 2 * far && seen < K; k++) {
                     const int c = own + ((k & 1) ? (k + 1) / 2 : -(k / 2));
                     if (c < c_lo || c > c_hi) continue;
-                    prefetch(c);
-                    seen += chunk(MfMax{}, c, -1, ev_j0, ev_j1);
+                    seen += chunk32(c, ev_j0, ev_j1);
                 }
                 mx = fmaxf(mx, __int_as_float(mf_other_half(__float_as_int(mx))));   // each lane saw half of the rows
                 // fewer than K usable candidates in the whole event: everything is collected
@@ -441,14 +599,6 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
                 const int f = d < DH ? d : 4 + d - DH;
                 qlo[d] = mf_wave_min_f(ing ? qx[f] : INFINITY);
                 qhi[d] = mf_wave_max_f(ing ? qx[f] : -INFINITY);
-            }
-            // float16 scale: every candidate within the bound of its query has |c'| sigma <= 120
-            {
-                const float need = mf_wave_max_f(ing ? sqrtf(qn) + sqrtf(bound) : 0.f);
-                const float want = 120.f / fmaxf(need, 1e-30f);
-                sig = __uint_as_float(min(max(__float_as_uint(want) & 0xff800000u, 0x20000000u), 0x5f000000u));   // 2^e, e in [-63, 63]
-#pragma unroll
-                for (int j = 0; j < DH; j++) osig[j] = o[j] * sig;
             }
             if (pass == 0) {
                 // B: histogram over the seed chunks
@@ -470,13 +620,14 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
                 }
                 hsc = 0.f;
             } else {
-                // D: collect everything whose screening value is below the bound (units of the accumulators: sigma^2)
-                set_b16(1.f);
-                thr = (ing && !over) ? bound * sig * sig * (1.0f + 0x1p-20f) : -INFINITY;
+                // D: collect everything whose screening value is below the bound
+                collecting = true;
+                cur_g = -1;
                 prefetch(s_lo);
                 for (int c = s_lo; c <= s_hi; c++) chunk(MfCollect{}, c, c < s_hi ? c + 1 : -1, ev_j0, ev_j1);
                 scan_event(MfCollect{}, ev_j0, ev_j1, s_lo, s_hi, bound, qlo, qhi);
                 thr = -INFINITY;
+                collecting = false;
             }
         }
     }
@@ -493,6 +644,7 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
         const long long orig_q = (long long)a.order[self];
         const int n0 = fgc_readlane_i(n_own, qq), n1 = fgc_readlane_i(n_own, qq + 32);
         const int c = n0 + n1;                    // <= CAP
+        const int evb = fgc_readlane_i(ev_base, qq);
         if (STATS) n_coll += (unsigned)c;
         float qs_[8];
 #pragma unroll
@@ -505,7 +657,7 @@ __global__ __launch_bounds__(64) void k_knn_mf(KnnArgs a)
             const int e = s * 64 + lane;
             const bool have = e < c;
             const int r = e < n0 ? e : CAP - 1 - (e - n0);
-            const int id = have ? (int)col[(r << 5) + qq] : self;
+            const int id = have ? evb + (int)col[(r << 5) + qq] : self;
             const float4 c0 = sp4[(size_t)id * 2], c1 = sp4[(size_t)id * 2 + 1];
             const float cx[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
             float df = qs_[0] - cx[0];
@@ -663,7 +815,7 @@ static int mf_column_height(int K) { return max(64, (K + max(K >> 1, 32) + 7) & 
 template <int D, int NSEG, int PS, bool STATS> static int launch_mf_t(const KnnArgs &a, hipStream_t s)
 {
     const int blocks = (int)fgc_cdiv(a.n, MF_QT);
-    const size_t lds = (size_t)32 * a.pool_cap * 4 + (size_t)NSEG * 64 * 8;
+    const size_t lds = (size_t)32 * a.pool_cap * 2 + (size_t)NSEG * 64 * 8;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)k_knn_mf<D, NSEG, PS, STATS>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);

@@ -48,7 +48,10 @@ extern "C" {
                                 sort every row before comparing, tests/test_binned_select_knn.py:90-91); saves the
                                 per-query sort */
 #define FGC_KNN_NO_MATRIX 4  /* keep the vector-unit search where the library would screen the candidates on the
-                                matrix cores (5 to 8 coordinates, K <= 256); same neighbours, for comparison runs */
+                                matrix cores (5 to 8 coordinates, K <= 256, events of at most 65535 points and of a
+                                size at which bounding boxes thin out little); same neighbours, for comparison runs */
+#define FGC_KNN_FORCE_MATRIX 8 /* screen on the matrix cores wherever that search can run (5 to 8 coordinates, K <= 256,
+                                events of at most 65535 points), whatever the event sizes; for comparison runs */
 
 #define FGC_STATUS_WORDS 4
 /* bits of d_status[0] */
@@ -122,7 +125,7 @@ int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t ld_coords,
  *                 :67-82) or passes the user's n_bins
  *   d_direction   int64 [n_vert] or NULL (0: only neighbour, 1: only query,
  *                 2: neither; binned_select_knn_cuda_kernel.cu:120-122,194-196)
- *   tf_compat     bit set of FGC_KNN_TF_COMPAT, FGC_KNN_ANY_ORDER and FGC_KNN_NO_MATRIX (0 or 1 as before: rows
+ *   tf_compat     bit set of FGC_KNN_TF_COMPAT, FGC_KNN_ANY_ORDER, FGC_KNN_NO_MATRIX and FGC_KNN_FORCE_MATRIX (0 or 1 as before: rows
  *                 by distance)
  *   d_idx         out int64 [n_vert, K]: slot 0 the query itself, then its
  *                 K-1 nearest points of the same event by increasing distance
@@ -133,7 +136,10 @@ int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t ld_coords,
  *   d_stats       optional uint64[8] device counters, accumulated: [0] distance
  *                 evaluations, [1] candidate chunks visited, [2] pool prunes
  *                 ([3..7] only in debug builds with -DFGC_KNN_COUNTERS: box
- *                 tests, appends, spans, bisection steps); NULL to skip.  A call
+ *                 tests, appends, spans, bisection steps; when the search ran
+ *                 on the matrix cores: [3] queries it handed to the vector
+ *                 search, [5] candidates it collected for the others, and
+ *                 [0] counts screened pairs); NULL to skip.  A call
  *                 with d_stats runs a second build of the search kernels that carries
  *                 the counters and is slower (time a call without)
  */
