@@ -572,22 +572,31 @@ def cpu_reference_full(w, K, n):
 
 
 def cpu_baseline(w, K, n, budget_s):
-    """The CPU restatement of the reference algorithm (oracle/, the checker)
-    timed single-threaded, like the reference's CPU kernel, on every s-th query
-    of the same bin-sorted workload; s is chosen from a short probe so that the
-    run takes about `budget_s` seconds."""
+    """The reference's CPU search on this box's host cores, on a bounded sample of the workload's queries.
+
+    Headline (`kind: "reference"`): the reference's own kernel (binned_select_knn_cpu.cpp:56-208, compiled unmodified
+    into oracle/_ref), single-threaded as it is written, with the reference's own grid.  The kernel has no query
+    stride, but it skips a query whose direction flag is 0 and still takes that point as a neighbour
+    (binned_select_knn_cpu.cpp:80-83,157-160): all points but every s-th get flag 0, the sampled ones a flag that
+    allows both roles, and use_direction is set - the unmodified kernel then searches the sampled queries among ALL
+    points.  The rows of the sampled queries are compared with the restatement's (oracle/, `kind: "port"`), which is
+    timed on the same queries; where oracle/_ref is not built the restatement is the headline.
+    Returns (one-core entry, all-cores entry of the restatement with OpenMP over the queries)."""
+    import numpy as np
     from oracle import oracle as O
     s = O.sorted_space(w["coords"], w["row_splits"], K)
     args = (s["scoords"], s["sbin"], s["sdbin"], s["bin_boundaries"], s["n_bins"], s["bin_width"], K)
     stride = max(1, n // 2000)
     t0 = time.perf_counter()
-    _, _, ev, _ = O.knn_sorted(*args, n_threads=1, query_stride=stride)
+    O.knn_sorted(*args, n_threads=1, query_stride=stride)
     probe = time.perf_counter() - t0
     per_query = probe / max(1, (n + stride - 1) // stride)
-    want = max(1, int(budget_s / max(per_query, 1e-9)))
+    have_ref = O.ref_lib() is not None
+    # the reference's kernel takes about twice the restatement's time per query; both run on the same sample
+    want = max(1, int(budget_s / max((2.2 if have_ref else 1.0) * per_query, 1e-9)))
     stride2 = max(1, n // want)
     t0 = time.perf_counter()
-    _, _, ev2, _ = O.knn_sorted(*args, n_threads=1, query_stride=stride2)
+    pi, pd, ev2, _ = O.knn_sorted(*args, n_threads=1, query_stride=stride2)
     t = time.perf_counter() - t0
     nq = (n + stride2 - 1) // stride2
     cpu_model = "unknown"
@@ -602,11 +611,29 @@ def cpu_baseline(w, K, n, budget_s):
     import torch
     host = {"cpu_model": cpu_model, "nproc": os.cpu_count(), "usable_cores": len(os.sched_getaffinity(0)),
             "torch_threads": torch.get_num_threads()}
-    one = {"value": round(nq / t, 1), "unit": "queries/s", "cores": 1, "kind": "port", "host": host,
-           "sample": "every %d-th query of the bin-sorted workload (%d queries, %.1f s, %d distance "
-                     "evaluations); kNN search kernel only, binning and sort excluded" % (stride2, nq, t, ev2)}
-    # the same restatement with OpenMP over the queries on the cores this process may use (the reference's CPU
-    # kernel itself is single-threaded); a second, shorter sample
+    sample = ("every %d-th query of the bin-sorted workload (%d queries) among all %d points, n_bins %s; kNN search "
+              "kernel only, binning and sort excluded" % (stride2, nq, n, [int(v) for v in s["n_bins"]]))
+    port = {"value": round(nq / t, 1), "unit": "queries/s", "cores": 1, "kind": "port", "seconds": round(t, 1),
+            "distance_evaluations": int(ev2)}
+    if have_ref:
+        tiny = O.sorted_space(w["coords"][:256], np.array([0, 256], dtype=np.int64), 4)   # loads the library, untimed
+        O.knn_sorted(tiny["scoords"], tiny["sbin"], tiny["sdbin"], tiny["bin_boundaries"], tiny["n_bins"],
+                     tiny["bin_width"], 4, use_ref=True)
+        direction = np.zeros(n, dtype=np.int64)           # 0: may only be a neighbour
+        direction[::stride2] = 3                          # neither 0, 1 nor 2: query and neighbour
+        t0 = time.perf_counter()
+        ri, rd, _, _ = O.knn_sorted(*args, sdirection=direction, use_ref=True)
+        t_ref = time.perf_counter() - t0
+        same = bool((ri[::stride2] == pi[::stride2]).all() and (rd[::stride2] == pd[::stride2]).all())
+        one = {"value": round(nq / t_ref, 1), "unit": "queries/s", "cores": 1, "kind": "reference", "host": host,
+               "seconds": round(t_ref, 1),
+               "sample": sample + "; the reference's compiled kernel, unmodified, the other queries switched off "
+                                  "through its direction flags",
+               "rows_identical_to_port_on_the_sample": same, "port_on_the_same_sample": port}
+    else:
+        one = dict(port, host=host, sample=sample + "; oracle/_ref is not built on this machine")
+    # the restatement with OpenMP over the queries on the cores this process may use (the reference's CPU kernel
+    # itself is single-threaded); a second, shorter sample
     threads = max(1, min(O.lib().fgc_oracle_max_threads(), len(os.sched_getaffinity(0)), 16))
     stride3 = max(1, stride2 // max(1, threads // 2))
     t0 = time.perf_counter()
@@ -615,25 +642,6 @@ def cpu_baseline(w, K, n, budget_s):
     nq3 = (n + stride3 - 1) // stride3
     many = {"value": round(nq3 / t3, 1), "unit": "queries/s", "cores": threads, "kind": "port",
             "sample": "every %d-th query (%d queries, %.1f s), OpenMP over queries" % (stride3, nq3, t3)}
-    # the reference's own compiled CPU kernel (oracle/_ref, when it was built) has no query stride, so it is timed
-    # on the same generator at a tenth of the points, next to the restatement on identical inputs: the ratio says
-    # how far the restatement's rate stands for the reference's
-    if O.ref_lib() is not None and w["name"].startswith("cfg4"):
-        from fastgraphcompute_amd import workloads
-        ws = workloads.CONFIGS["cfg4"](0.1)
-        ss = O.sorted_space(ws["coords"], ws["row_splits"], K)
-        sargs = (ss["scoords"], ss["sbin"], ss["sdbin"], ss["bin_boundaries"], ss["n_bins"], ss["bin_width"], K)
-        ns = ws["coords"].shape[0]
-        t0 = time.perf_counter()
-        ri, rd, _, _ = O.knn_sorted(*sargs, use_ref=True)
-        t_ref = time.perf_counter() - t0
-        t0 = time.perf_counter()
-        pi, pd, _, _ = O.knn_sorted(*sargs, n_threads=1)
-        t_port = time.perf_counter() - t0
-        one["reference_check"] = {
-            "sample": "cfg4 generator at scale 0.1 (%d points), all queries, one core" % ns,
-            "reference_queries_per_s": round(ns / t_ref, 1), "port_queries_per_s": round(ns / t_port, 1),
-            "identical_results": bool((ri == pi).all() and (rd == pd).all())}
     return one, many
 
 

@@ -233,3 +233,27 @@ def test_against_compiled_reference_kernels(oracle):
         r2 = oracle.bin_by_coordinates(np.ascontiguousarray(w["coords"][:, :Db]), w["row_splits"], None, 17, use_ref=True)
         for x, y in zip(r1, r2):
             np.testing.assert_array_equal(x, y)
+
+
+def test_reference_kernel_on_a_query_sample(oracle):
+    """How bench.py times the reference's own kernel on a bounded sample: direction flag 0 (may only be a neighbour)
+    for all points but every s-th, a flag outside 0..2 for the sampled ones, use_direction on
+    (binned_select_knn_cpu.cpp:80-83,157-160).  The sampled rows equal a search without any flags."""
+    if oracle.ref_lib() is None:
+        pytest.skip("oracle/_ref not built (needs the reference checkout)")
+    from fastgraphcompute_amd.workloads import cfg2_blobs_4events
+    w = cfg2_blobs_4events(0.03)
+    K = 12
+    s = oracle.sorted_space(w["coords"], w["row_splits"], K)
+    args = (s["scoords"], s["sbin"], s["sdbin"], s["bin_boundaries"], s["n_bins"], s["bin_width"], K)
+    n = w["coords"].shape[0]
+    full_i, full_d, _, _ = oracle.knn_sorted(*args, use_ref=True)
+    stride = 7
+    direction = np.zeros(n, dtype=np.int64)
+    direction[::stride] = 3
+    samp_i, samp_d, _, _ = oracle.knn_sorted(*args, sdirection=direction, use_ref=True)
+    np.testing.assert_array_equal(samp_i[::stride], full_i[::stride])
+    np.testing.assert_array_equal(samp_d[::stride], full_d[::stride])
+    port_i, port_d, _, _ = oracle.knn_sorted(*args, n_threads=1, query_stride=stride)
+    np.testing.assert_array_equal(port_i[::stride], full_i[::stride])
+    np.testing.assert_array_equal(port_d[::stride], full_d[::stride])
