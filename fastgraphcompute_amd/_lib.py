@@ -43,6 +43,8 @@ SIGNATURES = {
                                                         _i32, _vp, _vp]),
     "fgc_gravnet_aggregate_bwd_ld_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _i32, _vp, _i32,
                                                         _vp, _i64, _i32, _i32, _vp, _vp]),
+    "fgc_noalloc_init": (ctypes.c_int, []),
+    "fgc_gravnet_aggregate_bwd_sorted_supported": (ctypes.c_int, [_i64, _i32, _i32, _i32, _i32]),
     "fgc_gravnet_aggregate_bwd_sorted_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _vp, _i32,
                                                             _vp, _i64, _i32, _i32, _vp, _vp]),
     "fgc_index_replacer_i64": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _vp]),

@@ -161,7 +161,17 @@ def knn_grad(grad_distsq: torch.Tensor, idx: torch.Tensor, coords: torch.Tensor,
     with torch.cuda.device(x.device):
         _lib.check(L.fgc_binned_select_knn_grad_f32(_lib.ptr(g), _lib.ptr(ii), _lib.ptr(x), _lib.ptr(out), n, K, D,
                                                     _lib.ptr(order), _lib.ptr(status), _lib.stream_ptr()))
+    _raise_on_bad_index(status, "binned_select_knn_grad")
     return out
+
+
+def _raise_on_bad_index(status: torch.Tensor, what: str):
+    """For the ops that follow neighbour indices supplied by the caller: with config.sync_checks, wait for the op's
+    status word and raise if an index named a row that does not exist (the kernels treat such an entry as an empty
+    slot and set FGC_ST_BAD_INDEX; the reference would read out of bounds).  The autograd paths, whose indices come
+    from the library's own search, do not wait."""
+    if config.sync_checks and (int(status[0].item()) & _lib.ST_BAD_INDEX):
+        raise IndexError("%s: a neighbour index is not below the number of rows" % what)
 
 
 _PINNED = threading.local()
@@ -461,9 +471,12 @@ class _GravNetAggregate(torch.autograd.Function):
         fmean = torch.empty((n, P), dtype=torch.float32, device=f.device)
         fmax = torch.empty((n, P), dtype=torch.float32, device=f.device)
         argmax = torch.empty((n, P), dtype=torch.int32, device=f.device)
+        status = torch.zeros(4, dtype=torch.int32, device=f.device)
         with torch.cuda.device(f.device):
-            _lib.check(L.fgc_gravnet_aggregate_fwd_f32(_lib.ptr(ii), _lib.ptr(d), _lib.ptr(f), _lib.ptr(fmean),
-                                                       _lib.ptr(fmax), _lib.ptr(argmax), n, K, P, _lib.stream_ptr()))
+            _lib.check(L.fgc_gravnet_aggregate_fwd_ld_f32(_lib.ptr(ii), _lib.ptr(d), _lib.ptr(f), P, f.shape[0],
+                                                          _lib.ptr(fmean), _lib.ptr(fmax), P, _lib.ptr(argmax), n, K, P,
+                                                          _lib.ptr(status), _lib.stream_ptr()))
+        _raise_on_bad_index(status, "gravnet_aggregate")
         ctx.save_for_backward(ii, d, f, argmax)
         ctx.set_materialize_grads(False)
         return fmean, fmax
@@ -538,7 +551,8 @@ class _GravNetLayerCore(torch.autograd.Function):
             g_feat = torch.zeros_like(feat)
             g_dsq = torch.empty_like(dist)
             with torch.cuda.device(feat.device):
-                if config.tile_aggregation_backward and K <= 64 and 8 < P <= 64 and nbr_sorted.shape[0] == n:
+                if config.tile_aggregation_backward and nbr_sorted.shape[0] == n and \
+                        L.fgc_gravnet_aggregate_bwd_sorted_supported(n, K, P, P, P):
                     # rows that are neighbours in the search's sorted order share their targets: combined on chip
                     _lib.check(L.fgc_gravnet_aggregate_bwd_sorted_f32(
                         _lib.ptr(nbr_sorted), _lib.ptr(order), _lib.ptr(dist), _lib.ptr(feat), P, _lib.ptr(argmax),

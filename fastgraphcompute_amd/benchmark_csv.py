@@ -48,7 +48,9 @@ def main(argv=None):
         for n in a.sizes:
             for k in a.k:
                 for d in a.dims:
-                    t = time_call(n, d, min(k, 256), a.repeat)
+                    if not 1 <= k <= 1024:
+                        raise SystemExit("benchmark_csv: k must be in 1..1024 (the library's limit), got %d" % k)
+                    t = time_call(n, d, k, a.repeat)                 # the K that is written is the K that is timed
                     w.writerow([float(n), float(k), float(d), t, float(a.repeat)])
                     f.flush()
                     print("size %d k %d dimension %d: %.3f ms" % (n, k, d, t), flush=True)

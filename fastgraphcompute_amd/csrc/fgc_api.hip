@@ -5,7 +5,7 @@
 #include <cstdlib>
 #include <mutex>
 
-extern "C" int fgc_version(void) { return 100; }
+extern "C" int fgc_version(void) { return 101; }
 
 extern "C" const char *fgc_error_string(int code)
 {
@@ -14,6 +14,8 @@ extern "C" const char *fgc_error_string(int code)
     case FGC_EINVAL: return "invalid argument (shape, size or row splits)";
     case FGC_ENOSPACE: return "workspace too small";
     case FGC_EUNSUPPORTED: return "Unsupported number of binning dimensions.";
+    case FGC_ESHAPE:
+        return "shape outside what this specialised entry point handles; the general entry point takes every shape";
     case FGC_ETOOLARGE:
         return "input needs more scratch memory than the fixed area of the no-allocation entry point "
                "(FGC_NOALLOC_SCRATCH_BYTES); use fgc_binned_select_knn_f32 with a workspace of the caller";
@@ -232,12 +234,11 @@ int knn_search(float tau0, int32_t *d_nbr_sorted, int64_t n_vert, int32_t n_coor
     a.grp = c.w.with_sp ? (const float *)(ws + c.w.grp) : nullptr;
     a.mfstat = c.w.with_sp ? (const unsigned *)(ws + c.w.mfstat) : nullptr;
     a.redo = nullptr;
-    // many coordinates: candidates screened on the matrix cores (a radius bound keeps the vector search, which
-    // culls by it from the first bin row on)
     // Many coordinates and events that the bounding boxes cannot thin out: the matrix-core search.  Measured on
     // uniform and clustered points with 1 000 to 65 000 points per event: it wins up to about 1024 * 4^(D - 5)
     // points per event (twice that from K = 64 on), where the size is the one a typical point sees, sum n_e^2 / n.
-    // It stores candidates as 16-bit positions inside their event, so no event may exceed 65535 points.
+    // It stores candidates as 16-bit positions inside their event, so no event may exceed 65535 points.  A search
+    // with a radius bound keeps the vector search, which culls by the bound from the first bin row on.
     int64_t largest_event = 0;
     double sum_sq = 0;
     for (int r = 1; r < n_rs; r++) {
@@ -259,6 +260,8 @@ int knn_search(float tau0, int32_t *d_nbr_sorted, int64_t n_vert, int32_t n_coor
     return a.stats ? fgc_launch_knn_stats(a, (hipStream_t)stream) : fgc_launch_knn(a, (hipStream_t)stream);
 }
 
+}  // namespace
+
 extern "C" int fgc_binned_knn_export_order_i32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
                                                int32_t n_rs, int32_t K, int32_t n_bin_dims,
                                                const int64_t *n_bins, int32_t with_direction, const void *d_ws,
@@ -274,7 +277,6 @@ extern "C" int fgc_binned_knn_export_order_i32(int64_t n_vert, int32_t n_coords,
     sorted_buffers(c, (char *)const_cast<void *>(d_ws), &skeys, &order);
     return fgc_copy_u32(d_order_out, order, n_vert, (hipStream_t)stream);
 }
-}  // namespace
 
 extern "C" int fgc_binned_knn_search_f32(int64_t n_vert, int32_t n_coords, const int64_t *row_splits_host,
                                          int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
@@ -352,6 +354,15 @@ int scratch_address(void **out)
     return FGC_OK;
 }
 }  // namespace
+
+// Looks the scratch address of the current device up ahead of time, so that the first
+// fgc_binned_select_knn_noalloc_f32 on that device does no symbol lookup (and no lazy load of the code object): a
+// caller that captures the entry point into a HIP graph calls this once per device before it starts capturing.
+extern "C" int fgc_noalloc_init(void)
+{
+    void *ws = nullptr;
+    return scratch_address(&ws);
+}
 
 extern "C" int fgc_binned_select_knn_noalloc_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
                                                  const int64_t *d_row_splits, const int64_t *row_splits_host,

@@ -935,6 +935,13 @@ __global__ __launch_bounds__(GT_WAVES * 64) void k_gravnet_bwd_tile(
         rows_am[(tw0 + t) * PW + pl] = (unsigned char)am;
     }
 
+    // Step 1b reads, with lane = feature, what step 1a wrote to LDS with lane = slot: other lanes of the same
+    // wavefront.  The LDS queue of a wavefront keeps its order, so no block barrier is needed, but the compiler must
+    // not move a read above a write of another lane: a wavefront-level fence pins the order.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
     // ---- 1b. dot products for grad_distsq: lane = feature, QPW rows at a time, eight slots per step; the feature
     //      gathers of the next step are requested before the current one is reduced ----
     const int n_grp = (K + 7) >> 3;
@@ -1149,6 +1156,17 @@ extern "C" int fgc_gravnet_aggregate_bwd_ld_f32(const int64_t *d_idx, const floa
     return FGC_OK;
 }
 
+extern "C" int fgc_gravnet_aggregate_bwd_sorted_supported(int64_t n_vert, int32_t K, int32_t P, int32_t ld_feat,
+                                                          int32_t ld_grad_feat)
+{
+    if (K > 64 || P > 64 || P <= 8) return 0;
+    // 32-bit byte offsets of the feature and gradient rows, formed with a 24-bit multiply
+    if (n_vert >= (1 << 24) || ld_feat >= (1 << 22) || (uint64_t)n_vert * (uint64_t)ld_feat * 4ull >= 0xffffffffull ||
+        ld_grad_feat >= (1 << 22) || (uint64_t)n_vert * (uint64_t)ld_grad_feat * 4ull >= 0xffffffffull)
+        return 0;
+    return 1;
+}
+
 extern "C" int fgc_gravnet_aggregate_bwd_sorted_f32(const int32_t *d_nbr_sorted, const int32_t *d_order,
                                                     const float *d_distsq, const float *d_feat, int32_t ld_feat,
                                                     const int32_t *d_argmax, const float *d_grad_fmean,
@@ -1157,11 +1175,7 @@ extern "C" int fgc_gravnet_aggregate_bwd_sorted_f32(const int32_t *d_nbr_sorted,
                                                     int32_t K, int32_t P, int32_t *d_status, void *stream)
 {
     if (n_vert < 0 || K < 1 || P < 1 || ld_feat < P || ld_grad < P || ld_grad_feat < P) return FGC_EINVAL;
-    if (K > 64 || P > 64 || P <= 8 || n_vert >= (1ll << 31) - 1) return FGC_EUNSUPPORTED;
-    // 32-bit byte offsets of the feature and gradient rows, formed with a 24-bit multiply
-    if (n_vert >= (1 << 24) || ld_feat >= (1 << 22) || (uint64_t)n_vert * (uint64_t)ld_feat * 4ull >= 0xffffffffull ||
-        ld_grad_feat >= (1 << 22) || (uint64_t)n_vert * (uint64_t)ld_grad_feat * 4ull >= 0xffffffffull)
-        return FGC_EUNSUPPORTED;
+    if (!fgc_gravnet_aggregate_bwd_sorted_supported(n_vert, K, P, ld_feat, ld_grad_feat)) return FGC_ESHAPE;
     if (n_vert == 0) return FGC_OK;
     if (!d_nbr_sorted || !d_order || !d_distsq || !d_feat || !d_argmax || !d_grad_fmean || !d_grad_fmax ||
         !d_grad_feat || !d_grad_distsq)

@@ -33,6 +33,8 @@ extern "C" {
 #define FGC_ENOSPACE (-2)    /* workspace too small                           */
 #define FGC_EUNSUPPORTED (-3)/* e.g. number of binned dims outside 1..5       */
 #define FGC_ETOOLARGE (-4)   /* input exceeds the fixed scratch of a no-allocation entry point */
+#define FGC_ESHAPE (-5)      /* a shape outside what a specialised entry point handles (its comment says which
+                                general entry point takes every shape)          */
 
 #define FGC_MAX_BIN_DIMS 5
 #define FGC_MAX_K 1024       /* neighbours per query the kNN kernels support; the reference's loops take any
@@ -170,6 +172,11 @@ int fgc_binned_select_knn_f32(const float *d_coords, int64_t n_vert, int32_t n_c
  *   - The current device at the call must be the one the pointers belong to.
  */
 #define FGC_NOALLOC_SCRATCH_BYTES (32u << 20)
+/* Optional, once per device with that device current: looks up the device address of the scratch array (a symbol
+ * lookup, which may load the library's code object) so that the entry point itself does neither on its first call.
+ * Call it before capturing fgc_binned_select_knn_noalloc_f32 into a HIP graph; without it the first call per device
+ * does the lookup itself and must therefore happen outside a capture.  No counterpart in the reference. */
+int fgc_noalloc_init(void);
 int fgc_binned_select_knn_noalloc_f32(const float *d_coords, int64_t n_vert, int32_t n_coords,
                                       const int64_t *d_row_splits, const int64_t *row_splits_host,
                                       int32_t n_rs, int32_t K, int32_t n_bin_dims, const int64_t *n_bins,
@@ -329,7 +336,12 @@ int fgc_gravnet_aggregate_bwd_ld_f32(const int64_t *d_idx, const float *d_distsq
  * the original order): the feature gradients of 16 consecutive sorted rows, which share most of their neighbours,
  * are combined on chip, so that one row update per distinct target of the tile reaches memory instead of one per
  * (point, slot) pair.  Same results as fgc_gravnet_aggregate_bwd_ld_f32 up to the order of the float sums.
- * Supports K <= 64 and 8 < P <= 64 (FGC_EUNSUPPORTED otherwise: use the entry point above). */
+ * Supports K <= 64, 8 < P <= 64, fewer than 2^24 points, rows of fewer than 2^22 floats and matrices of less than
+ * 4 GiB (24-bit row arithmetic, 32-bit byte offsets); FGC_ESHAPE otherwise: fgc_gravnet_aggregate_bwd_ld_f32 takes
+ * every shape.  fgc_gravnet_aggregate_bwd_sorted_supported returns 1 for exactly the shapes this entry point takes,
+ * so that a caller can choose without trying. */
+int fgc_gravnet_aggregate_bwd_sorted_supported(int64_t n_vert, int32_t K, int32_t P, int32_t ld_feat,
+                                               int32_t ld_grad_feat);
 int fgc_gravnet_aggregate_bwd_sorted_f32(const int32_t *d_nbr_sorted, const int32_t *d_order, const float *d_distsq,
                                          const float *d_feat, int32_t ld_feat, const int32_t *d_argmax,
                                          const float *d_grad_fmean, const float *d_grad_fmax, int32_t ld_grad,

@@ -159,3 +159,25 @@ def test_integration_shim_compiles_against_the_header():
             cmd += ["-I", inc]
         r = subprocess.run(cmd + [path], capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stderr[-4000:]
+
+
+def test_tile_backward_predicate_and_entry_point_agree():
+    """GravNetOp's backward asks fgc_gravnet_aggregate_bwd_sorted_supported before it takes the tile kernel; the
+    entry point must reject (FGC_ESHAPE, nothing launched) exactly the shapes the predicate turns down - among them
+    layers of 2^24 points and more, which fit this GPU - and name the general entry point in its message."""
+    import ctypes
+    from fastgraphcompute_amd import _lib
+    L = _lib.lib()
+    p = ctypes.c_void_p(4096)
+    assert b"general entry point" in L.fgc_error_string(-5)
+    cases = [(100, 40, 32, 32, 32), (100, 64, 64, 64, 64), (100, 65, 32, 32, 32), (100, 40, 8, 8, 8), (100, 40, 65, 65, 65),
+             ((1 << 24) - 1, 40, 32, 32, 32), (1 << 24, 40, 32, 32, 32), (20_000_000, 40, 32, 32, 32),
+             (1 << 23, 40, 32, 128, 32), (1 << 23, 40, 32, 32, 128), (1000, 40, 32, 1 << 22, 32), (0, 40, 32, 32, 32)]
+    for n, K, P, ldf, ldg in cases:
+        ok = L.fgc_gravnet_aggregate_bwd_sorted_supported(n, K, P, ldf, ldg)
+        if ok and n > 0:
+            continue          # a supported shape would launch: only the rejections can be tried without a GPU
+        rc = L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, ldf, p, p, p, P, p, ldg, p, n, K, P, None, None)
+        assert (rc == -5) == (not ok), (n, K, P, ldf, ldg, ok, rc)
+    assert L.fgc_gravnet_aggregate_bwd_sorted_supported(1 << 24, 40, 32, 32, 32) == 0
+    assert L.fgc_gravnet_aggregate_bwd_sorted_supported((1 << 24) - 1, 40, 32, 32, 32) == 1

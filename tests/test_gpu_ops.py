@@ -404,8 +404,8 @@ def test_gravnet_backward_in_sorted_space_rejects_unsupported_shapes():
     fake = ctypes_ptr = None
     import ctypes
     p = ctypes.c_void_p(4096)
-    assert L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, 32, p, p, p, 32, p, 32, p, 100, 65, 32, None, None) == -3
-    assert L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, 8, p, p, p, 8, p, 8, p, 100, 8, 8, None, None) == -3
+    assert L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, 32, p, p, p, 32, p, 32, p, 100, 65, 32, None, None) == -5
+    assert L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, 8, p, p, p, 8, p, 8, p, 100, 8, 8, None, None) == -5
     assert L.fgc_gravnet_aggregate_bwd_sorted_f32(p, p, p, p, 16, p, p, p, 32, p, 32, p, 100, 8, 32, None, None) == -1
 
 

@@ -34,3 +34,22 @@ def test_on_device_feeds_knn():
     assert torch.equal(strict_batch_from_row_splits(rs), b)
     idx, _ = binned_select_knn(4, torch.rand(500, 3, device="cuda"), rs)
     assert bool((idx[:300] < 300).all()) and bool((idx[300:] >= 300).all())
+
+
+@pytest.mark.gpu
+def test_benchmark_csv_rows(tmp_path):
+    """The timing sweep writes the columns the reference's published table is keyed on (size, k, dimension, fgc_time,
+    count; graphing/master_data.csv, written by performance/generate_faiss_performance.py:95-135 and the scripts
+    next to it) and times the K it writes - also beyond 256 neighbours."""
+    import csv
+    from fastgraphcompute_amd import benchmark_csv
+    out = tmp_path / "t.csv"
+    benchmark_csv.main(["--out", str(out), "--sizes", "3000", "--dims", "3", "6", "--k", "300", "--repeat", "2"])
+    rows = list(csv.reader(open(out)))
+    assert rows[0] == ["size", "k", "dimension", "fgc_time", "count"]
+    assert len(rows) == 3
+    for r, d in zip(rows[1:], (3.0, 6.0)):
+        assert float(r[0]) == 3000.0 and float(r[1]) == 300.0 and float(r[2]) == d and float(r[4]) == 2.0
+        assert 0.0 < float(r[3]) < 1e4
+    with pytest.raises(SystemExit):
+        benchmark_csv.main(["--out", str(out), "--sizes", "3000", "--dims", "3", "--k", "2000", "--repeat", "1"])

@@ -91,3 +91,52 @@ def test_noalloc_rejects_inputs_beyond_its_fixed_scratch():
     with pytest.raises(RuntimeError, match="scratch"):
         _lib.check(rc)
     assert int((idx != -7).sum().item()) == 0          # nothing was launched
+
+
+def test_noalloc_allocates_nothing_and_can_be_captured():
+    """After fgc_noalloc_init (the scratch address looked up ahead of time) the entry point leaves the device's free
+    memory unchanged, and it can be captured into a HIP graph: every replay, with eager work and synchronisations in
+    between, equals the eager call on the same input."""
+    from fastgraphcompute_amd import _lib
+    L = _lib.lib()
+    assert L.fgc_noalloc_init() == 0
+    n, D, K = 30000, 3, 24
+    rs_host = [0, 11000, n]
+    rs = torch.tensor(rs_host, dtype=torch.int64, device="cuda")
+    rsa, nb = _lib.host_i64(rs_host), _lib.host_i64([4, 4, 4])
+    coords = torch.rand(n, D, device="cuda")
+    idx = torch.empty((n, K), dtype=torch.int64, device="cuda")
+    dist = torch.empty((n, K), dtype=torch.float32, device="cuda")
+    status = torch.zeros(4, dtype=torch.int32, device="cuda")
+
+    def enqueue():
+        _lib.check(L.fgc_binned_select_knn_noalloc_f32(_lib.ptr(coords), n, D, _lib.ptr(rs), rsa, 3, K, 3, nb, None, 0,
+                                                       _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(status),
+                                                       _lib.stream_ptr()))
+
+    enqueue()
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    enqueue()
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, "the call changed the device's free memory"
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        enqueue()
+    ws_bytes = L.fgc_binned_select_knn_workspace_bytes(n, D, 3, nb, 3, K)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    ref_i, ref_d = torch.empty_like(idx), torch.empty_like(dist)
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    for rep in range(3):
+        coords.copy_(torch.rand(n, D, device="cuda", generator=gen) * (rep + 1))
+        g.replay()
+        torch.cuda.synchronize()
+        got_i, got_d = idx.clone(), dist.clone()
+        _lib.check(L.fgc_binned_select_knn_f32(_lib.ptr(coords), n, D, _lib.ptr(rs), rsa, 3, K, 3, nb, None, 0,
+                                               _lib.ptr(ref_i), _lib.ptr(ref_d), _lib.ptr(status), None, _lib.ptr(ws),
+                                               ws_bytes, _lib.stream_ptr()))              # eager work in between
+        torch.cuda.synchronize()
+        assert torch.equal(got_d, ref_d) and torch.equal(got_i, ref_i), "replay %d differs" % rep
