@@ -174,25 +174,33 @@ extern "C" int fgc_binned_knn_prepare_ld_f32(const float *d_coords, int64_t n_ve
     float *sc = (float *)(ws + w.sc);
     unsigned char *sdir = d_direction ? (unsigned char *)(ws + w.sdir) : nullptr;
 
-    rc = fgc_bin_geometry_f32(d_coords, n_vert, ld_coords, n_bin_dims, 2, n_bins, 1, 0.f, 0, geom, d_status,
-                              ws + w.partial, fgc_bin_geometry_workspace_bytes(n_vert), stream);
-    if (rc) return rc;
-    rc = fgc_launch_bin_keys(d_coords, (int)n_vert, ld_coords, n_bin_dims, c.sub_bits, geom, d_row_splits, n_rs,
-                             keys, d_status, s);
-    if (rc) return rc;
+    float *spp = w.with_sp ? (float *)(ws + w.sp) : nullptr;
     uint32_t *skeys = nullptr, *order = nullptr;
-    rc = fgc_sort_keys(keys, vals, n_vert, c.key_bits, ws + w.sort, s, &skeys, &order);
-    if (rc) return rc;
-    uint32_t *skeys2, *order2;
-    sorted_buffers(c, ws, &skeys2, &order2);
-    if (skeys2 != skeys || order2 != order) return FGC_EINVAL;  // internal layout mismatch
-    rc = fgc_launch_bin_boundaries(skeys, (int)n_vert, c.sub_bits * n_bin_dims, (int)c.B, bb, s);
-    if (rc) return rc;
-    rc = fgc_launch_gather_sorted(d_coords, ld_coords, order, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir,
-                                  w.with_sp ? (float *)(ws + w.sp) : nullptr, fgc_knn_sp_half(n_coords), s);
-    if (rc) return rc;
-    rc = fgc_launch_chunk_boxes(sc, (int)n_vert, n_coords, w.ldc, (float *)(ws + w.box_lo),
-                                (float *)(ws + w.box_hi), (float *)(ws + w.sbox_lo), (float *)(ws + w.sbox_hi), s);
+    if (fgc_sort_fused_fits(n_vert)) {
+        // up to a few hundred thousand points: one launch per sort pass, the geometry record derived by the key kernel
+        rc = fgc_keys_and_sort_fused(d_coords, (int)n_vert, ld_coords, n_bin_dims, n_bins, c.sub_bits, c.key_bits,
+                                     d_row_splits, n_rs, (float *)(ws + w.partial), geom, keys, vals, ws + w.sort,
+                                     d_status, s, &skeys, &order);
+        if (rc) return rc;
+    } else {
+        rc = fgc_bin_geometry_f32(d_coords, n_vert, ld_coords, n_bin_dims, 2, n_bins, 1, 0.f, 0, geom, d_status,
+                                  ws + w.partial, fgc_bin_geometry_workspace_bytes(n_vert), stream);
+        if (rc) return rc;
+        rc = fgc_launch_bin_keys(d_coords, (int)n_vert, ld_coords, n_bin_dims, c.sub_bits, geom, d_row_splits, n_rs,
+                                 keys, d_status, s);
+        if (rc) return rc;
+        rc = fgc_sort_keys(keys, vals, n_vert, c.key_bits, ws + w.sort, s, &skeys, &order);
+        if (rc) return rc;
+    }
+    {
+        uint32_t *skeys2, *order2;
+        sorted_buffers(c, ws, &skeys2, &order2);
+        if (skeys2 != skeys || order2 != order) return FGC_EINVAL;  // internal layout mismatch
+    }
+    rc = fgc_launch_prepare_tail(d_coords, ld_coords, order, skeys, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir,
+                                 spp, fgc_knn_sp_half(n_coords), (float *)(ws + w.box_lo), (float *)(ws + w.box_hi),
+                                 (float *)(ws + w.sbox_lo), (float *)(ws + w.sbox_hi), c.sub_bits * n_bin_dims,
+                                 (int)c.B, bb, s);
     if (rc || !w.with_sp) return rc;
     return fgc_launch_mf_operands((const float *)(ws + w.sp), (const float *)(ws + w.box_lo),
                                   (const float *)(ws + w.box_hi), (int)n_vert, n_coords, w.ldc, (float *)(ws + w.grp),

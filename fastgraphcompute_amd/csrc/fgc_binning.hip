@@ -42,15 +42,23 @@ int fgc_copy_u32(void *dst, const void *src, int64_t n_words, hipStream_t s)
     return FGC_OK;
 }
 
+// minimum / maximum over the 64 lanes, in every lane: four DPP steps inside each row of 16 lanes, then the four
+// rows through scalar reads
 __device__ __forceinline__ float wave_min_f(float v)
 {
-    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, 64));
-    return v;
+    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true)));
+    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true)));
+    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true)));
+    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true)));
+    return fminf(fminf(fgc_readlane_f(v, 0), fgc_readlane_f(v, 16)), fminf(fgc_readlane_f(v, 32), fgc_readlane_f(v, 48)));
 }
 __device__ __forceinline__ float wave_max_f(float v)
 {
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true)));
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true)));
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true)));
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true)));
+    return fmaxf(fmaxf(fgc_readlane_f(v, 0), fgc_readlane_f(v, 16)), fmaxf(fgc_readlane_f(v, 32), fgc_readlane_f(v, 48)));
 }
 
 // ---------------------------------------------------------------------------
@@ -59,9 +67,12 @@ __device__ __forceinline__ float wave_max_f(float v)
 #define RANGE_BLOCKS_MAX 1024
 
 // partial[blk][0..4] = min, [5..9] = max, [10] = non-finite seen (as float 0/1)
+// (also clears `zero_words` words at `zero`: the digit tables of the sort that follows on a small input)
 __global__ __launch_bounds__(256) void k_range_partial(const float *__restrict__ coords, int64_t n,
-                                                       int ld, int nbd, float *__restrict__ partial)
+                                                       int ld, int nbd, float *__restrict__ partial,
+                                                       uint32_t *__restrict__ zero, int zero_words)
 {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < zero_words; i += gridDim.x * blockDim.x) zero[i] = 0u;
     float mn[FGC_MAX_BIN_DIMS], mx[FGC_MAX_BIN_DIMS];
     int bad = 0;
 #pragma unroll
@@ -98,33 +109,14 @@ __global__ __launch_bounds__(256) void k_range_partial(const float *__restrict__
     }
 }
 
-// One wave: reduce the partials and derive the geometry record.  Arithmetic
-// order as the reference's tensor ops: (max - min), +1 where the range is
-// zero, +1e-3, width = max_d(range_d / n_bins_d)  [or n_bins from a width].
-__global__ __launch_bounds__(64) void k_geometry(const float *__restrict__ partial, int nblk, int nbd,
-                                                 int mode, int nb_given, float bw_in, int pre_norm,
-                                                 int nb0, int nb1, int nb2, int nb3, int nb4,
-                                                 float *__restrict__ geom, int *__restrict__ status)
+// The geometry record from the per-dimension range (one thread).  Arithmetic order as the reference's tensor ops:
+// (max - min), +1 where the range is zero, +1e-3, width = max_d(range_d / n_bins_d)  [or n_bins from a width].
+__device__ inline void geometry_record(const float (&mn)[FGC_MAX_BIN_DIMS], const float (&mx)[FGC_MAX_BIN_DIMS], bool bad,
+                                       int nbd, int mode, int nb_given, float bw_in, int pre_norm,
+                                       const int (&nb_in)[FGC_MAX_BIN_DIMS], float *__restrict__ geom,
+                                       int *__restrict__ status)
 {
-    const int lane = fgc_lane();
-    float mn[FGC_MAX_BIN_DIMS], mx[FGC_MAX_BIN_DIMS];
-    float bad = 0.f;
-#pragma unroll
-    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) { mn[d] = INFINITY; mx[d] = -INFINITY; }
-    for (int b = lane; b < nblk; b += 64) {
-#pragma unroll
-        for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
-            mn[d] = fminf(mn[d], partial[b * 11 + d]);
-            mx[d] = fmaxf(mx[d], partial[b * 11 + 5 + d]);
-        }
-        bad = fmaxf(bad, partial[b * 11 + 10]);
-    }
-#pragma unroll
-    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) { mn[d] = wave_min_f(mn[d]); mx[d] = wave_max_f(mx[d]); }
-    bad = wave_max_f(bad);
-    if (lane != 0) return;
-    const int nb_in[FGC_MAX_BIN_DIMS] = {nb0, nb1, nb2, nb3, nb4};
-    int flags = bad > 0.f ? FGC_ST_NONFINITE : 0;
+    int flags = bad ? FGC_ST_NONFINITE : 0;
     float rng[FGC_MAX_BIN_DIMS];
     float bw = bw_in;
     for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
@@ -163,6 +155,45 @@ __global__ __launch_bounds__(64) void k_geometry(const float *__restrict__ parti
     if (status && flags) atomicOr(&status[0], flags);
 }
 
+// One block: reduce the partials and derive the geometry record.
+__global__ __launch_bounds__(256) void k_geometry(const float *__restrict__ partial, int nblk, int nbd,
+                                                  int mode, int nb_given, float bw_in, int pre_norm,
+                                                  int nb0, int nb1, int nb2, int nb3, int nb4,
+                                                  float *__restrict__ geom, int *__restrict__ status)
+{
+    __shared__ float s_red[4][11];
+    const int lane = fgc_lane(), wv = threadIdx.x >> 6;
+    float mn[FGC_MAX_BIN_DIMS], mx[FGC_MAX_BIN_DIMS];
+    float bad = 0.f;
+#pragma unroll
+    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) { mn[d] = INFINITY; mx[d] = -INFINITY; }
+    for (int b = threadIdx.x; b < nblk; b += 256) {
+#pragma unroll
+        for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
+            mn[d] = fminf(mn[d], partial[b * 11 + d]);
+            mx[d] = fmaxf(mx[d], partial[b * 11 + 5 + d]);
+        }
+        bad = fmaxf(bad, partial[b * 11 + 10]);
+    }
+#pragma unroll
+    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
+        const float a = wave_min_f(mn[d]), b = wave_max_f(mx[d]);
+        if (lane == 0) { s_red[wv][d] = a; s_red[wv][5 + d] = b; }
+    }
+    bad = wave_max_f(bad);
+    if (lane == 0) s_red[wv][10] = bad;
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+#pragma unroll
+    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
+        mn[d] = fminf(fminf(s_red[0][d], s_red[1][d]), fminf(s_red[2][d], s_red[3][d]));
+        mx[d] = fmaxf(fmaxf(s_red[0][5 + d], s_red[1][5 + d]), fmaxf(s_red[2][5 + d], s_red[3][5 + d]));
+    }
+    bad = fmaxf(fmaxf(s_red[0][10], s_red[1][10]), fmaxf(s_red[2][10], s_red[3][10]));
+    const int nb_in[FGC_MAX_BIN_DIMS] = {nb0, nb1, nb2, nb3, nb4};
+    geometry_record(mn, mx, bad > 0.f, nbd, mode, nb_given, bw_in, pre_norm, nb_in, geom, status);
+}
+
 extern "C" size_t fgc_bin_geometry_workspace_bytes(int64_t n_vert)
 {
     (void)n_vert;
@@ -191,9 +222,9 @@ extern "C" int fgc_bin_geometry_f32(const float *d_coords, int64_t n_vert, int32
     int nblk = (int)fgc_cdiv(n_vert, 256 * 4);
     if (nblk > RANGE_BLOCKS_MAX) nblk = RANGE_BLOCKS_MAX;
     hipLaunchKernelGGL(k_range_partial, dim3(nblk), dim3(256), 0, s, d_coords, n_vert, (int)ld_coords,
-                       (int)n_bin_dims, (float *)d_ws);
+                       (int)n_bin_dims, (float *)d_ws, (uint32_t *)nullptr, 0);
     FGC_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_geometry, dim3(1), dim3(64), 0, s, (const float *)d_ws, nblk, (int)n_bin_dims,
+    hipLaunchKernelGGL(k_geometry, dim3(1), dim3(256), 0, s, (const float *)d_ws, nblk, (int)n_bin_dims,
                        (int)mode, (int)n_bins_given, bin_width_in, (int)pre_normalized, nb[0], nb[1],
                        nb[2], nb[3], nb[4], d_geom, d_status);
     FGC_LAUNCH_CHECK();
@@ -308,15 +339,10 @@ extern "C" int fgc_bin_points_f32(const float *d_coords, int64_t n_vert, int32_t
 // run of 64 points has a tight bounding box wherever it starts); it never changes
 // which bin a point belongs to.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void k_bin_keys(const float *__restrict__ coords, int n, int ld, int nbd,
-                                                  int sub_bits, const float *__restrict__ geom,
-                                                  const int64_t *__restrict__ rs, int n_rs,
-                                                  uint32_t *__restrict__ keys, int *__restrict__ status)
+// key of point v (its coordinates at `row`, its event `ev`)
+__device__ inline uint32_t knn_sort_key(const float *__restrict__ row, const BinGeom &g, int nbd, int sub_bits, int ev,
+                                        int &clamped)
 {
-    int v = blockIdx.x * blockDim.x + threadIdx.x;
-    if (v >= n) return;
-    BinGeom g = load_geom(geom);
-    int clamped = 0;
     uint32_t f = 0, stride = 1;
     int sub[FGC_MAX_BIN_DIMS];
     const int smax = (1 << sub_bits) - 1;
@@ -324,7 +350,7 @@ __global__ __launch_bounds__(256) void k_bin_keys(const float *__restrict__ coor
     for (int d = FGC_MAX_BIN_DIMS - 1; d >= 0; d--) {
         sub[d] = 0;
         if (d < nbd) {
-            const float x = coords[(int64_t)v * ld + d];
+            const float x = row[d];
             int b = bin_of(x, g.mn[d], g.bw, g.nb[d], clamped);
             f += (uint32_t)b * stride;
             stride *= (uint32_t)g.nb[d];
@@ -333,8 +359,7 @@ __global__ __launch_bounds__(256) void k_bin_keys(const float *__restrict__ coor
             sub[d] = min(max((int)(fr * (float)(smax + 1)), 0), smax);
         }
     }
-    f += (uint32_t)event_of(rs, n_rs, v) * stride;
-    if (clamped && status) atomicOr(&status[0], FGC_ST_CLAMPED);
+    f += (uint32_t)ev * stride;
 #ifndef FGC_MORTON_KEYS
     // sub-cell coordinates -> transposed Hilbert index (Skilling's in-place transform: undo the excess work of
     // the Gray code from the most significant level down, then Gray-encode), so that interleaving the bits
@@ -371,7 +396,20 @@ __global__ __launch_bounds__(256) void k_bin_keys(const float *__restrict__ coor
 #pragma unroll
         for (int d = 0; d < FGC_MAX_BIN_DIMS; d++)
             if (d < nbd) code = (code << 1) | (uint32_t)((sub[d] >> l) & 1);
-    keys[v] = (f << (sub_bits * nbd)) | code;
+    return (f << (sub_bits * nbd)) | code;
+}
+
+__global__ __launch_bounds__(256) void k_bin_keys(const float *__restrict__ coords, int n, int ld, int nbd,
+                                                  int sub_bits, const float *__restrict__ geom,
+                                                  const int64_t *__restrict__ rs, int n_rs,
+                                                  uint32_t *__restrict__ keys, int *__restrict__ status)
+{
+    int v = blockIdx.x * blockDim.x + threadIdx.x;
+    if (v >= n) return;
+    BinGeom g = load_geom(geom);
+    int clamped = 0;
+    keys[v] = knn_sort_key(coords + (int64_t)v * ld, g, nbd, sub_bits, event_of(rs, n_rs, v), clamped);
+    if (clamped && status) atomicOr(&status[0], FGC_ST_CLAMPED);
 }
 
 // ---------------------------------------------------------------------------
@@ -553,6 +591,7 @@ __global__ __launch_bounds__(256) void k_rs_scatter(const uint32_t *__restrict__
 size_t fgc_sort_workspace_bytes(int64_t n)
 {
     int64_t nblk = fgc_cdiv(n > 0 ? n : 1, RS_MIN_TILE);   // the smallest tile has the most blocks
+    if (n <= 32768) nblk *= 3;                             // three digit tables of the one-launch passes
     return fgc_align((size_t)n * 4) * 2 /* ping-pong keys / vals */ + fgc_align((size_t)nblk * 256 * 4) +
            fgc_align(256 * 4) /* digit totals */;
 }
@@ -597,54 +636,6 @@ int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void 
     return FGC_OK;
 }
 
-// bin_boundaries[b] = first sorted position whose bin is >= b, for b in [0, n_bins_total]: one binary search
-// per bin (long runs of empty bins, e.g. around outliers, cost nothing extra)
-__global__ __launch_bounds__(256) void k_bin_boundaries(const uint32_t *__restrict__ skeys, int n, int shift,
-                                                        int n_bins_total, int *__restrict__ bb)
-{
-    const int b = blockIdx.x * blockDim.x + threadIdx.x;
-    if (b > n_bins_total) return;
-    int lo = 0, hi = n;
-    while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if ((long long)(skeys[mid] >> shift) < (long long)b) lo = mid + 1; else hi = mid;
-    }
-    bb[b] = lo;
-}
-
-// sorted structure-of-arrays coordinates: sc[d * ldc + i] = coords[order[i]][d]
-__global__ __launch_bounds__(256) void k_gather_sorted(const float *__restrict__ coords, int ld_in,
-                                                       const uint32_t *__restrict__ order, int n, int D,
-                                                       int ldc, float *__restrict__ sc,
-                                                       const int64_t *__restrict__ direction,
-                                                       unsigned char *__restrict__ sdir, float4 *__restrict__ sp,
-                                                       int sp_half)
-{
-    int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (sp && i >= n && i < ldc) {           // padding rows of the last chunk
-        sp[(int64_t)i * 2] = make_float4(0.f, 0.f, 0.f, 0.f);
-        sp[(int64_t)i * 2 + 1] = make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-    if (i >= n) return;
-    uint32_t o = order[i];
-    if (sp) {
-        float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int d = 0; d < D; d++) {
-            const float x = coords[(int64_t)o * ld_in + d];
-            sc[(int64_t)d * ldc + i] = x;
-            if (d < 2 * sp_half) r[d < sp_half ? d : 4 + d - sp_half] = x;
-        }
-        sp[(int64_t)i * 2] = make_float4(r[0], r[1], r[2], r[3]);
-        sp[(int64_t)i * 2 + 1] = make_float4(r[4], r[5], r[6], r[7]);
-    } else {
-        for (int d = 0; d < D; d++) sc[(int64_t)d * ldc + i] = coords[(int64_t)o * ld_in + d];
-    }
-    if (sdir) {
-        int64_t v = direction[o];
-        sdir[i] = (unsigned char)((v >= 0 && v <= 2) ? v : 3);
-    }
-}
-
 int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, int sub_bits, const float *d_geom,
                         const int64_t *d_rs, int n_rs, uint32_t *d_keys, int *d_status, hipStream_t s)
 {
@@ -654,68 +645,416 @@ int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, int sub_b
     return FGC_OK;
 }
 
-int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int shift, int n_bins_total, int *bb, hipStream_t s)
+// ---------------------------------------------------------------------------
+// Up to FS_MAX_N points (a few dozen tiles) the sort needs ONE launch per pass instead of three, and the geometry record none of its
+// own: launches of a few microseconds each otherwise dominate the preparation of a few thousand points - the
+// typical event of the reference's tests.
+//   * k_bin_keys_geom: every block reduces the range partials itself (a few hundred records) and derives the
+//     geometry record in LDS (block 0 also stores it); it adds its keys' lowest digits to the first digit table.
+//   * k_rs_pass: a digit table holds, tile by tile, how many keys of the tile have each digit (table[tile][digit]).
+//     Every block sums the table's rows itself - the rows before its own tile and all of them - instead of reading
+//     a scan another launch made; while it writes a key to its sorted position it adds the key's NEXT digit to
+//     the next pass's table at the tile that position lies in; and it clears its row of a third table for the pass
+//     after that.  Integer atomic adds only: the tables, hence the order, do not depend on timing.
+// No block waits for another inside a launch.
+// ---------------------------------------------------------------------------
+#define FS_MAX_N 32768
+#define FS_CH 4
+#define FS_TILE (256 * FS_CH)
+#define FS_TILE_SHIFT 10
+
+__global__ __launch_bounds__(256) void k_bin_keys_geom(const float *__restrict__ coords, int n, int ld, int nbd,
+                                                       int sub_bits, const float *__restrict__ partial, int npart,
+                                                       int nb0, int nb1, int nb2, int nb3, int nb4,
+                                                       float *__restrict__ geom_out, const int64_t *__restrict__ rs,
+                                                       int n_rs, uint32_t *__restrict__ keys,
+                                                       int *__restrict__ status, uint32_t *__restrict__ table0)
 {
-    hipLaunchKernelGGL(k_bin_boundaries, dim3((unsigned)fgc_cdiv((int64_t)n_bins_total + 1, 256)), dim3(256), 0, s,
-                       skeys, n, shift, n_bins_total, bb);
-    FGC_LAUNCH_CHECK();
-    return FGC_OK;
+    __shared__ float s_red[4][11];
+    __shared__ float s_geom[FGC_GEOM_FLOATS];
+    __shared__ uint32_t s_h[256];
+    const int t = threadIdx.x, lane = fgc_lane(), wv = t >> 6;
+    // this thread's point and its event first: the loads travel while the geometry record is made
+    const int v = blockIdx.x * 256 + t;
+    float x[FGC_MAX_BIN_DIMS];
+#pragma unroll
+    for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) x[d] = (v < n && d < nbd) ? coords[(int64_t)v * ld + d] : 0.f;
+    const int ev = v < n ? event_of(rs, n_rs, v) : 0;
+    {
+        float mn[FGC_MAX_BIN_DIMS], mx[FGC_MAX_BIN_DIMS];
+        float bad = 0.f;
+#pragma unroll
+        for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) { mn[d] = INFINITY; mx[d] = -INFINITY; }
+        for (int b = t; b < npart; b += 256) {
+#pragma unroll
+            for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
+                mn[d] = fminf(mn[d], partial[b * 11 + d]);
+                mx[d] = fmaxf(mx[d], partial[b * 11 + 5 + d]);
+            }
+            bad = fmaxf(bad, partial[b * 11 + 10]);
+        }
+#pragma unroll
+        for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
+            const float a = wave_min_f(mn[d]), b = wave_max_f(mx[d]);
+            if (lane == 0) { s_red[wv][d] = a; s_red[wv][5 + d] = b; }
+        }
+        bad = wave_max_f(bad);
+        if (lane == 0) s_red[wv][10] = bad;
+        s_h[t] = 0;
+        __syncthreads();
+        if (t == 0) {
+#pragma unroll
+            for (int d = 0; d < FGC_MAX_BIN_DIMS; d++) {
+                mn[d] = fminf(fminf(s_red[0][d], s_red[1][d]), fminf(s_red[2][d], s_red[3][d]));
+                mx[d] = fmaxf(fmaxf(s_red[0][5 + d], s_red[1][5 + d]), fmaxf(s_red[2][5 + d], s_red[3][5 + d]));
+            }
+            bad = fmaxf(fmaxf(s_red[0][10], s_red[1][10]), fmaxf(s_red[2][10], s_red[3][10]));
+            const int nb_in[FGC_MAX_BIN_DIMS] = {nb0, nb1, nb2, nb3, nb4};
+            geometry_record(mn, mx, bad > 0.f, nbd, 2, 1, 0.f, 0, nb_in, s_geom, blockIdx.x == 0 ? status : nullptr);
+            if (blockIdx.x == 0)
+                for (int d = 0; d < FGC_GEOM_FLOATS; d++) geom_out[d] = s_geom[d];
+        }
+        __syncthreads();
+    }
+    if (v < n) {
+        const BinGeom g = load_geom(s_geom);
+        int clamped = 0;
+        const uint32_t key = knn_sort_key(x, g, nbd, sub_bits, ev, clamped);
+        keys[v] = key;
+        if (clamped && status) atomicOr(&status[0], FGC_ST_CLAMPED);
+        atomicAdd(&s_h[key & 255u], 1u);
+    }
+    __syncthreads();
+    // the 256 keys of a block lie in one tile of the sort
+    if (s_h[t]) atomicAdd(&table0[(size_t)((blockIdx.x * 256) >> FS_TILE_SHIFT) * 256 + t], s_h[t]);
 }
 
-int fgc_launch_gather_sorted(const float *coords, int ld_in, const uint32_t *order, int n, int D, int ldc, float *sc,
-                             const int64_t *direction, unsigned char *sdir, float *sp, int sp_half, hipStream_t s)
+__global__ __launch_bounds__(256) void k_rs_pass(const uint32_t *__restrict__ keys_in,
+                                                 const uint32_t *__restrict__ vals_in, uint32_t *__restrict__ keys_out,
+                                                 uint32_t *__restrict__ vals_out, int n, int shift, int nblk,
+                                                 const uint32_t *__restrict__ table, uint32_t *__restrict__ table_next,
+                                                 uint32_t *__restrict__ table_clear)
 {
-    hipLaunchKernelGGL(k_gather_sorted, dim3((unsigned)fgc_cdiv(sp ? ldc : n, 256)), dim3(256), 0, s, coords, ld_in,
-                       order, n, D, ldc, sc, direction, sdir, (float4 *)sp, sp_half);
-    FGC_LAUNCH_CHECK();
-    return FGC_OK;
-}
-
-// axis-aligned bounding box of every 64 consecutive sorted points, all D coordinates:
-// box_lo[d * n_chunks + c], box_hi[d * n_chunks + c]
-__global__ __launch_bounds__(256) void k_chunk_boxes(const float *__restrict__ sc, int n, int D, int ldc,
-                                                     int n_chunks, float *__restrict__ box_lo,
-                                                     float *__restrict__ box_hi)
-{
-    const int lane = fgc_lane();
-    const int c = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
-    if (c >= n_chunks) return;
-    const int j = c * 64 + lane;
-    for (int d = 0; d < D; d++) {
-        const float x = (j < n) ? sc[(size_t)d * ldc + j] : NAN;
-        const float lo = wave_min_f((j < n) ? x : INFINITY);
-        const float hi = wave_max_f((j < n) ? x : -INFINITY);
-        if (lane == 0) { box_lo[(size_t)d * n_chunks + c] = lo; box_hi[(size_t)d * n_chunks + c] = hi; }
+    __shared__ uint32_t s_cnt[4][256];
+    __shared__ uint32_t s_gbase[256];
+    __shared__ uint32_t s_ws[4], s_ws2[4];
+    __shared__ int s_const;
+    __shared__ uint32_t s_key[FS_TILE], s_val[FS_TILE];
+    const int t = threadIdx.x, lane = fgc_lane(), wv = t >> 6, blk = blockIdx.x;
+    if (table_clear) table_clear[(size_t)blk * 256 + t] = 0u;
+    const int tile0 = blk * FS_TILE;
+    const int n_tile = min(FS_TILE, n - tile0);
+    const int next_shift = shift + 8;
+    const int base = tile0 + wv * (FS_TILE / 4);
+    uint32_t key[FS_CH], val[FS_CH];
+#pragma unroll
+    for (int c = 0; c < FS_CH; c++) {
+        const int i = base + c * 64 + lane;
+        key[c] = i < n ? keys_in[i] : 0u;
+        val[c] = i < n ? (vals_in ? vals_in[i] : (uint32_t)i) : 0u;
+    }
+    // digit t: keys in the tiles before this one, keys in all tiles
+    uint32_t before = 0, total = 0;
+    {
+        int b = 0;
+        for (; b + 16 <= nblk; b += 16) {
+            uint32_t c[16];
+#pragma unroll
+            for (int k = 0; k < 16; k++) c[k] = table[(size_t)(b + k) * 256 + t];
+#pragma unroll
+            for (int k = 0; k < 16; k++) { total += c[k]; before += (b + k < blk) ? c[k] : 0u; }
+        }
+        uint32_t c[16];
+#pragma unroll
+        for (int k = 0; k < 16; k++) c[k] = b + k < nblk ? table[(size_t)(b + k) * 256 + t] : 0u;
+#pragma unroll
+        for (int k = 0; k < 16; k++) { total += c[k]; before += (b + k < blk) ? c[k] : 0u; }
+    }
+    uint32_t incl = total;
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t u = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += u;
+    }
+    if (t == 0) s_const = 0;
+    if (lane == 63) s_ws[wv] = incl;
+    __syncthreads();
+    uint32_t first = incl - total;                 // sorted position of the first key with digit t
+    for (int k = 0; k < wv; k++) first += s_ws[k];
+    if (total == (uint32_t)n) s_const = 1;         // every key has this digit: the pass is the identity
+    volatile uint32_t *cnt = s_cnt[wv];
+    for (int i = lane; i < 256; i += 64) cnt[i] = 0;
+    __syncthreads();
+    if (s_const) {
+        for (int c = 0; c < FS_CH; c++) {
+            const int i = base + c * 64 + lane;
+            const bool valid = i < n;
+            if (valid) { keys_out[i] = key[c]; vals_out[i] = val[c]; }
+            if (table_next) {
+                const int nd = (int)((key[c] >> next_shift) & 255u);
+                const unsigned long long m = match_digit(nd, valid);
+                if (valid && fgc_mbcnt(m) == 0) atomicAdd(&table_next[(size_t)blk * 256 + nd], (uint32_t)__popcll(m));
+            }
+        }
+        return;
+    }
+    // per-wavefront digit counts
+#pragma unroll
+    for (int c = 0; c < FS_CH; c++) {
+        const bool valid = base + c * 64 + lane < n;
+        const int digit = (int)((key[c] >> shift) & 255u);
+        const unsigned long long m = match_digit(digit, valid);
+        if (valid && fgc_mbcnt(m) == 0) cnt[digit] = cnt[digit] + (uint32_t)__popcll(m);
+    }
+    __syncthreads();
+    // the tile in digit order inside LDS: start of every digit inside the tile, the running offsets of the four
+    // wavefronts on top of that, and the sorted position of the digit's first key of this tile minus that start
+    {
+        const uint32_t c0 = s_cnt[0][t], c1 = s_cnt[1][t], c2 = s_cnt[2][t], c3 = s_cnt[3][t];
+        const uint32_t tot = c0 + c1 + c2 + c3;
+        uint32_t in2 = tot;
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t u = __shfl_up(in2, o, 64);
+            if (lane >= o) in2 += u;
+        }
+        if (lane == 63) s_ws2[wv] = in2;
+        __syncthreads();
+        uint32_t loc = in2 - tot;
+        for (int k = 0; k < wv; k++) loc += s_ws2[k];
+        s_gbase[t] = first + before - loc;
+        s_cnt[0][t] = loc; s_cnt[1][t] = loc + c0; s_cnt[2][t] = loc + c0 + c1; s_cnt[3][t] = loc + c0 + c1 + c2;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < FS_CH; c++) {
+        const bool valid = base + c * 64 + lane < n;
+        const int digit = (int)((key[c] >> shift) & 255u);
+        const unsigned long long m = match_digit(digit, valid);
+        const int rank = fgc_mbcnt(m);
+        const uint32_t off = valid ? cnt[digit] : 0u;
+        if (valid && rank == 0) cnt[digit] = off + (uint32_t)__popcll(m);
+        if (valid) { s_key[off + (uint32_t)rank] = key[c]; s_val[off + (uint32_t)rank] = val[c]; }
+    }
+    __syncthreads();
+    for (int i = t; i < FS_TILE; i += 256) {
+        const bool valid = i < n_tile;
+        const uint32_t k = valid ? s_key[i] : 0u;
+        const uint32_t pos = valid ? s_gbase[(k >> shift) & 255u] + (uint32_t)i : 0u;
+        if (valid) { keys_out[pos] = k; vals_out[pos] = s_val[i]; }
+        if (table_next) {
+            // one add per (tile, digit) of the wavefront where its keys land in one tile (the usual case: a run of
+            // one digit), one per key otherwise
+            const int nd = (int)((k >> next_shift) & 255u);
+            const uint32_t dst = pos >> FS_TILE_SHIFT;
+            const bool mine = valid && dst == (uint32_t)__builtin_amdgcn_readfirstlane((int)dst);
+            const unsigned long long m = match_digit(nd, mine);
+            if (mine) {
+                if (fgc_mbcnt(m) == 0) atomicAdd(&table_next[(size_t)dst * 256 + nd], (uint32_t)__popcll(m));
+            } else if (valid) atomicAdd(&table_next[(size_t)dst * 256 + nd], 1u);
+        }
     }
 }
 
-// bounding box of every 64 consecutive chunks (aligned): sbox_lo[d * n_super + g], sbox_hi[d * n_super + g]
-__global__ __launch_bounds__(256) void k_super_boxes(const float *__restrict__ box_lo,
-                                                     const float *__restrict__ box_hi, int D, int n_chunks,
-                                                     int n_super, float *__restrict__ sbox_lo,
-                                                     float *__restrict__ sbox_hi)
+bool fgc_sort_fused_fits(int64_t n) { return n > 0 && n <= FS_MAX_N; }
+
+// range + geometry + keys + sort of a small input: 2 + passes launches.  `partial` as in fgc_bin_geometry_f32's
+// workspace, `d_sort_ws` as for fgc_sort_keys.
+int fgc_keys_and_sort_fused(const float *coords, int n, int ld, int nbd, const int64_t *n_bins, int sub_bits,
+                            int key_bits, const int64_t *rs, int n_rs, float *partial, float *geom, uint32_t *keys,
+                            uint32_t *vals, void *d_sort_ws, int *status, hipStream_t s, uint32_t **keys_sorted,
+                            uint32_t **vals_sorted)
 {
-    const int lane = fgc_lane();
-    const int g = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
-    if (g >= n_super) return;
-    const int c = g * 64 + lane;
-    for (int d = 0; d < D; d++) {
-        const float lo = wave_min_f(c < n_chunks ? box_lo[(size_t)d * n_chunks + c] : INFINITY);
-        const float hi = wave_max_f(c < n_chunks ? box_hi[(size_t)d * n_chunks + c] : -INFINITY);
-        if (lane == 0) { sbox_lo[(size_t)d * n_super + g] = lo; sbox_hi[(size_t)d * n_super + g] = hi; }
+    int nb[FGC_MAX_BIN_DIMS] = {1, 1, 1, 1, 1};
+    for (int d = 0; d < nbd; d++) {
+        if (n_bins[d] > 0x7fffffff) return FGC_EINVAL;
+        nb[d] = (int)n_bins[d];
+    }
+    char *w = (char *)d_sort_ws;
+    uint32_t *k_alt = (uint32_t *)w; w += fgc_align((size_t)n * 4);
+    uint32_t *v_alt = (uint32_t *)w; w += fgc_align((size_t)n * 4);
+    const int nblk = (int)fgc_cdiv(n, FS_TILE);
+    uint32_t *tab[3] = {(uint32_t *)w, (uint32_t *)w + (size_t)nblk * 256, (uint32_t *)w + (size_t)nblk * 512};
+    int npart = (int)fgc_cdiv(n, 256 * 4);
+    if (npart > RANGE_BLOCKS_MAX) npart = RANGE_BLOCKS_MAX;
+    hipLaunchKernelGGL(k_range_partial, dim3(npart), dim3(256), 0, s, coords, (int64_t)n, ld, nbd, partial, tab[0],
+                       nblk * 512);
+    FGC_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_bin_keys_geom, dim3((unsigned)fgc_cdiv(n, 256)), dim3(256), 0, s, coords, n, ld, nbd, sub_bits,
+                       partial, npart, nb[0], nb[1], nb[2], nb[3], nb[4], geom, rs, n_rs, keys, status, tab[0]);
+    FGC_LAUNCH_CHECK();
+    uint32_t *kin = keys, *vin = nullptr, *kout = k_alt, *vout = v_alt;
+    int passes = (key_bits + 7) / 8;
+    if (passes < 1) passes = 1;
+    for (int p = 0; p < passes; p++) {
+        hipLaunchKernelGGL(k_rs_pass, dim3(nblk), dim3(256), 0, s, kin, vin, kout, vout, n, p * 8, nblk, tab[p % 3],
+                           p + 1 < passes ? tab[(p + 1) % 3] : (uint32_t *)nullptr,
+                           p + 2 < passes ? tab[(p + 2) % 3] : (uint32_t *)nullptr);
+        FGC_LAUNCH_CHECK();
+        kin = kout; vin = vout;
+        if (kout == k_alt) { kout = keys; vout = vals; } else { kout = k_alt; vout = v_alt; }
+    }
+    *keys_sorted = kin;
+    *vals_sorted = vin;
+    return FGC_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The tail of the preparation in one launch: sorted coordinates (structure of arrays, optionally also as rows of 8
+// floats), direction flags, the bounding boxes of the chunks and of the groups of 64 chunks, and the bin
+// boundaries.  One block of 16 wavefronts per group of 64 chunks: wavefront w gathers chunks 4 w .. 4 w + 3 of the
+// group (lane = point; the loads of all four requested before the first is used) and reduces their boxes, the block
+// combines them into the group's box through LDS.  Bin boundaries (bb[b] = first sorted position whose bin is
+// >= b) from the same positions: where the bin changes between positions i - 1 and i, position i is the boundary
+// of every bin in between.
+// ---------------------------------------------------------------------------
+template <int DT>   // DT = D where the gather is unrolled for it, 0 = any D
+__global__ __launch_bounds__(1024) void k_prepare_tail(const float *__restrict__ coords, int ld_in,
+                                                       const uint32_t *__restrict__ order,
+                                                       const uint32_t *__restrict__ skeys, int n, int D_rt, int ldc,
+                                                       float *__restrict__ sc, const int64_t *__restrict__ direction,
+                                                       unsigned char *__restrict__ sdir, float4 *__restrict__ sp,
+                                                       int sp_half, float *__restrict__ box_lo,
+                                                       float *__restrict__ box_hi, float *__restrict__ sbox_lo,
+                                                       float *__restrict__ sbox_hi, int key_shift, int n_bins_total,
+                                                       int *__restrict__ bb)
+{
+    __shared__ float s_lo[16][16], s_hi[16][16];
+    const int D = DT ? DT : D_rt;
+    const int lane = fgc_lane(), wv = threadIdx.x >> 6;
+    const int n_chunks = ldc / 64, n_super = (n_chunks + 63) / 64;
+    const int g = blockIdx.x;                 // group of 64 chunks
+    const int c0 = g * 64 + wv * 4;
+    uint32_t o[4], key[4], keyp[4];
+    int64_t dirv[4];
+#pragma unroll
+    for (int cc = 0; cc < 4; cc++) {
+        const int i = (c0 + cc) * 64 + lane;
+        o[cc] = i < n ? order[i] : 0u;
+        key[cc] = i < n ? skeys[i] : 0u;
+        keyp[cc] = (i <= n && i > 0) ? skeys[i - 1] : 0u;
+    }
+    if (sdir) {
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++) dirv[cc] = (c0 + cc) * 64 + lane < n ? direction[o[cc]] : 0;
+    }
+    float glo[16], ghi[16];                   // this wavefront's share of the group's box, coordinate d in slot d (d < 16)
+#pragma unroll
+    for (int d = 0; d < 16; d++) { glo[d] = INFINITY; ghi[d] = -INFINITY; }
+    if (DT) {
+        float x[4][DT ? DT : 1];
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++)
+#pragma unroll
+            for (int d = 0; d < DT; d++) x[cc][d] = (c0 + cc) * 64 + lane < n ? coords[(int64_t)o[cc] * ld_in + d] : 0.f;
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++) {
+            const int c = c0 + cc, i = c * 64 + lane;
+            if (c >= n_chunks) break;
+            const bool in = i < n;
+            float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int d = 0; d < DT; d++) {
+                if (in) sc[(int64_t)d * ldc + i] = x[cc][d];
+                if (d < 2 * sp_half) r[d < sp_half ? d : 4 + d - sp_half] = x[cc][d];
+                const float lo = wave_min_f(in ? x[cc][d] : INFINITY), hi = wave_max_f(in ? x[cc][d] : -INFINITY);
+                if (lane == 0) { box_lo[(size_t)d * n_chunks + c] = lo; box_hi[(size_t)d * n_chunks + c] = hi; }
+                if (d < 16) { glo[d] = fminf(glo[d], lo); ghi[d] = fmaxf(ghi[d], hi); }
+            }
+            if (sp) {
+                sp[(int64_t)i * 2] = make_float4(r[0], r[1], r[2], r[3]);
+                sp[(int64_t)i * 2 + 1] = make_float4(r[4], r[5], r[6], r[7]);
+            }
+        }
+    } else {
+        for (int cc = 0; cc < 4; cc++) {
+            const int c = c0 + cc, i = c * 64 + lane;
+            if (c >= n_chunks) break;
+            const bool in = i < n;
+            float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            for (int d = 0; d < D; d++) {
+                const float x = in ? coords[(int64_t)o[cc] * ld_in + d] : 0.f;
+                if (in) sc[(int64_t)d * ldc + i] = x;
+                if (d < 2 * sp_half) r[d < sp_half ? d : 4 + d - sp_half] = x;
+                const float lo = wave_min_f(in ? x : INFINITY), hi = wave_max_f(in ? x : -INFINITY);
+                if (lane == 0) { box_lo[(size_t)d * n_chunks + c] = lo; box_hi[(size_t)d * n_chunks + c] = hi; }
+                if (d < 16) { glo[d] = fminf(glo[d], lo); ghi[d] = fmaxf(ghi[d], hi); }   // (coordinates 16 and up: below)
+            }
+            if (sp) {
+                sp[(int64_t)i * 2] = make_float4(r[0], r[1], r[2], r[3]);
+                sp[(int64_t)i * 2 + 1] = make_float4(r[4], r[5], r[6], r[7]);
+            }
+        }
+    }
+#pragma unroll
+    for (int cc = 0; cc < 4; cc++) {
+        const int i = (c0 + cc) * 64 + lane;
+        if (sdir && i < n) sdir[i] = (unsigned char)((dirv[cc] >= 0 && dirv[cc] <= 2) ? dirv[cc] : 3);
+        // bin boundaries
+        int b_from = 1, b_to = 0;                    // bins b_from .. b_to get the boundary `at`
+        int at = i;
+        if (i < n) {
+            b_from = i > 0 ? (int)(keyp[cc] >> key_shift) + 1 : 0;
+            b_to = (int)(key[cc] >> key_shift);
+        }
+        if (i == n) { b_from = n > 0 ? (int)(keyp[cc] >> key_shift) + 1 : 0; b_to = n_bins_total; at = n; }
+        if (b_to > n_bins_total) b_to = n_bins_total;    // (keys are made of valid bins; guards the store all the same)
+        // short runs by the lane itself, long ones (empty regions of the grid) by the whole wavefront
+        const bool longrun = b_to - b_from >= 8;
+        if (!longrun) for (int b = b_from; b <= b_to; b++) bb[b] = at;
+        unsigned long long m = fgc_ballot(longrun);
+        while (m) {
+            const int l = __builtin_ctzll(m);
+            m &= m - 1;
+            const int f = fgc_readlane_i(b_from, l), t2 = fgc_readlane_i(b_to, l), a = fgc_readlane_i(at, l);
+            for (int b = f + lane; b <= t2; b += 64) bb[b] = a;
+        }
+    }
+    if (lane < 16) {
+        float lo = INFINITY, hi = -INFINITY;
+#pragma unroll
+        for (int d = 0; d < 16; d++) if (lane == d) { lo = glo[d]; hi = ghi[d]; }
+        s_lo[wv][lane] = lo; s_hi[wv][lane] = hi;
+    }
+    __syncthreads();
+    if (g < n_super && threadIdx.x < min(D, 16)) {
+        float lo = INFINITY, hi = -INFINITY;
+        for (int w = 0; w < 16; w++) { lo = fminf(lo, s_lo[w][threadIdx.x]); hi = fmaxf(hi, s_hi[w][threadIdx.x]); }
+        sbox_lo[(size_t)threadIdx.x * n_super + g] = lo;
+        sbox_hi[(size_t)threadIdx.x * n_super + g] = hi;
+    }
+    if (D > 16 && g < n_super) {
+        // coordinates 16 and up (rare): from the chunk boxes this block has just written
+        for (int d = 16 + wv; d < D; d += 16) {
+            const int c = g * 64 + lane;
+            const float lo = wave_min_f(c < n_chunks ? box_lo[(size_t)d * n_chunks + c] : INFINITY);
+            const float hi = wave_max_f(c < n_chunks ? box_hi[(size_t)d * n_chunks + c] : -INFINITY);
+            if (lane == 0) { sbox_lo[(size_t)d * n_super + g] = lo; sbox_hi[(size_t)d * n_super + g] = hi; }
+        }
     }
 }
 
-int fgc_launch_chunk_boxes(const float *sc, int n, int D, int ldc, float *box_lo, float *box_hi, float *sbox_lo,
-                           float *sbox_hi, hipStream_t s)
+int fgc_launch_prepare_tail(const float *coords, int ld_in, const uint32_t *order, const uint32_t *skeys, int n, int D,
+                            int ldc, float *sc, const int64_t *direction, unsigned char *sdir, float *sp, int sp_half,
+                            float *box_lo, float *box_hi, float *sbox_lo, float *sbox_hi, int key_shift,
+                            int n_bins_total, int *bb, hipStream_t s)
 {
-    const int n_chunks = ldc / 64;
-    hipLaunchKernelGGL(k_chunk_boxes, dim3((unsigned)fgc_cdiv(n_chunks, 4)), dim3(256), 0, s, sc, n, D, ldc,
-                       n_chunks, box_lo, box_hi);
-    FGC_LAUNCH_CHECK();
-    const int n_super = (n_chunks + 63) / 64;
-    hipLaunchKernelGGL(k_super_boxes, dim3((unsigned)fgc_cdiv(n_super, 4)), dim3(256), 0, s,
-                       (const float *)box_lo, (const float *)box_hi, D, n_chunks, n_super, sbox_lo, sbox_hi);
+    // position n (the end of the last bin's run) must belong to a chunk some wavefront visits
+    const int n_super = ((n + 1 + 63) / 64 + 63) / 64;
+#define FGC_TAIL(DT)                                                                                                    \
+    hipLaunchKernelGGL(k_prepare_tail<DT>, dim3((unsigned)n_super), dim3(1024), 0, s, coords, ld_in, order, skeys, n, D, \
+                       ldc, sc, direction, sdir, (float4 *)sp, sp_half, box_lo, box_hi, sbox_lo, sbox_hi, key_shift,   \
+                       n_bins_total, bb)
+    switch (D) {
+    case 2: FGC_TAIL(2); break;
+    case 3: FGC_TAIL(3); break;
+    case 4: FGC_TAIL(4); break;
+    case 5: FGC_TAIL(5); break;
+    case 6: FGC_TAIL(6); break;
+    case 8: FGC_TAIL(8); break;
+    default: FGC_TAIL(0); break;
+    }
+#undef FGC_TAIL
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
+
+

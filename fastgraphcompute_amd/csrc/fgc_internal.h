@@ -7,13 +7,17 @@ int fgc_sort_keys(uint32_t *keys, uint32_t *vals, int64_t n, int key_bits, void 
                   uint32_t **keys_sorted, uint32_t **vals_sorted, bool vals_given = false);
 int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, int sub_bits, const float *d_geom,
                         const int64_t *d_rs, int n_rs, uint32_t *d_keys, int *d_status, hipStream_t s);
-int fgc_launch_bin_boundaries(const uint32_t *skeys, int n, int shift, int n_bins_total, int *bb, hipStream_t s);
-int fgc_launch_chunk_boxes(const float *sc, int n, int D, int ldc, float *box_lo, float *box_hi, float *sbox_lo,
-                           float *sbox_hi, hipStream_t s);
-// sp (optional): the sorted points once more as rows of 8 floats, two halves of 4 with `sp_half` coordinates each
-// (zero padded; rows n .. ldc - 1 are zero), for the matrix-core search
-int fgc_launch_gather_sorted(const float *coords, int ld_in, const uint32_t *order, int n, int D, int ldc, float *sc,
-                             const int64_t *direction, unsigned char *sdir, float *sp, int sp_half, hipStream_t s);
+// the tail of the preparation in one launch (sorted coordinates, boxes, bin boundaries), and for small inputs
+// everything before it (range, geometry, keys, sort) in two launches plus one per sort pass
+int fgc_launch_prepare_tail(const float *coords, int ld_in, const uint32_t *order, const uint32_t *skeys, int n, int D,
+                            int ldc, float *sc, const int64_t *direction, unsigned char *sdir, float *sp, int sp_half,
+                            float *box_lo, float *box_hi, float *sbox_lo, float *sbox_hi, int key_shift,
+                            int n_bins_total, int *bb, hipStream_t s);
+bool fgc_sort_fused_fits(int64_t n);
+int fgc_keys_and_sort_fused(const float *coords, int n, int ld, int nbd, const int64_t *n_bins, int sub_bits,
+                            int key_bits, const int64_t *rs, int n_rs, float *partial, float *geom, uint32_t *keys,
+                            uint32_t *vals, void *d_sort_ws, int *status, hipStream_t s, uint32_t **keys_sorted,
+                            uint32_t **vals_sorted);
 
 // kNN search over bin-sorted points (fgc_knn.hip)
 struct KnnArgs {

@@ -215,6 +215,20 @@ def test_tiny_inputs(oracle, n, K):
     check_knn_properties(gi, gd, coords, [0, n], K)
 
 
+@pytest.mark.parametrize("n", [1023, 1024, 1025, 4096, 4097, 32767, 32768, 32769, 40000])
+def test_sizes_around_the_preparation_paths(oracle, n):
+    """Inputs of up to 32768 points sort with one launch per pass (digit tables summed by every block), larger ones with
+    three; the bin boundaries come from the position after the last point, which lies in a chunk of its own when the
+    point count is a multiple of 64.  Four events of unequal size, one of them clustered (most bins empty)."""
+    rng = np.random.default_rng(n)
+    cuts = np.sort(rng.choice(np.arange(1, n), size=3, replace=False))
+    rs = np.concatenate([[0], cuts, [n]]).astype(np.int64)
+    coords = rng.random((n, 3)).astype(np.float32)
+    coords[rs[1]:rs[2]] = (0.5 + 0.01 * rng.standard_normal((rs[2] - rs[1], 3))).astype(np.float32)
+    gi, gd = _check(oracle, 10, coords, rs)
+    check_knn_properties(gi, gd, coords, rs, 10)
+
+
 def test_all_points_coincident(oracle):
     coords = np.full((700, 3), 0.25, dtype=np.float32)
     gi, gd = _gpu_knn(10, coords, [0, 300, 700])
