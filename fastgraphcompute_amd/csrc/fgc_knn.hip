@@ -733,22 +733,28 @@ template <int DT, int NSEG, int RD> static int launch_knn_t(const KnnArgs &a, hi
     return FGC_OK;
 }
 
+// Kernels with the coordinates in registers are built for the combinations of coordinate count and binned dimensions
+// that the two grid rules produce (the library's own grid bins min(D, 5) dimensions, the reference's rule 3 - or 2
+// for D = 2); any other combination (a caller's max_bin_dims) runs the variant that reads coordinates from memory.
 template <int NSEG, int RD> static int launch_knn_d(const KnnArgs &a, hipStream_t s)
 {
+    constexpr bool wide = RD == 2 || RD == 4;      // 3 or 5 binned dimensions
     switch (a.D) {
-    case 2: return launch_knn_t<2, NSEG, RD>(a, s);
-    case 3: return launch_knn_t<3, NSEG, RD>(a, s);
-    case 4: return launch_knn_t<4, NSEG, RD>(a, s);
-    case 5: return launch_knn_t<5, NSEG, RD>(a, s);
-    case 6: return launch_knn_t<6, NSEG, RD>(a, s);
-    case 7: return launch_knn_t<7, NSEG, RD>(a, s);
-    case 8: return launch_knn_t<8, NSEG, RD>(a, s);
+    case 2: if constexpr (RD == 1) return launch_knn_t<2, NSEG, RD>(a, s); break;
+    case 3: if constexpr (RD == 2) return launch_knn_t<3, NSEG, RD>(a, s); break;
+    case 4: if constexpr (RD == 2 || RD == 3) return launch_knn_t<4, NSEG, RD>(a, s); break;
+    case 5: if constexpr (wide) return launch_knn_t<5, NSEG, RD>(a, s); break;
+    case 6: if constexpr (wide) return launch_knn_t<6, NSEG, RD>(a, s); break;
+    case 7: if constexpr (wide) return launch_knn_t<7, NSEG, RD>(a, s); break;
+    case 8: if constexpr (wide) return launch_knn_t<8, NSEG, RD>(a, s); break;
     default: break;
     }
     // more coordinates: padded up to 12 or 16 registers per point (the padding contributes exact zeros),
     // beyond that read from memory per evaluation
-    if (a.D <= 12) return launch_knn_t<12, NSEG, RD>(a, s);
-    if (a.D <= 16) return launch_knn_t<16, NSEG, RD>(a, s);
+    if constexpr (wide) {
+        if (a.D > 8 && a.D <= 12) return launch_knn_t<12, NSEG, RD>(a, s);
+        if (a.D > 12 && a.D <= 16) return launch_knn_t<16, NSEG, RD>(a, s);
+    }
     return launch_knn_t<0, NSEG, RD>(a, s);
 }
 
