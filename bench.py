@@ -24,11 +24,29 @@ N_SIMD = 1024           # 256 compute units x 4 SIMDs; a VALU wavefront instruct
 GPU_CLOCK_HZ = 2.4e9    # MI355X peak engine clock (published); used only to turn instruction counts into a time share
 
 
+def kernel_source_hash():
+    """First 12 hex digits of the SHA-256 over the library's HIP sources and headers (names and contents, in name
+    order): the `src=` field of a `#bench-fact` line says which sources the profiled library was built from."""
+    import hashlib
+    cdir = os.path.join(ROOT, "fastgraphcompute_amd", "csrc")
+    h = hashlib.sha256()
+    try:
+        names = sorted(n for n in os.listdir(cdir) if n.endswith((".hip", ".h")))
+        for n in names + ["../../include/fgc_hip.h"]:
+            with open(os.path.join(cdir, n), "rb") as fh:
+                h.update(os.path.basename(n).encode() + b"\0" + fh.read() + b"\0")
+    except OSError:
+        return None
+    return h.hexdigest()[:12]
+
+
 def profile_facts():
     """Per-kernel figures that only a profiler run gives (HBM bytes per launch from FETCH_SIZE / WRITE_SIZE,
     VALU wavefront instructions per launch), read from the `#bench-fact` lines of the committed rocprofv3 summaries
-    under profiles/: {(kernel, workload): {key: value, "file": name}}.  Both are properties of the kernel and the
-    input, not of the run, so they are combined here with the kernel time measured live."""
+    under profiles/: {(kernel, workload): {key: value, "files": names, "src": source hashes}}.  Both are properties
+    of the kernel and the input, not of the run, so they are combined here with the kernel time measured live - as
+    long as the kernel is the one that was profiled: a line whose `src=` differs from the hash of the sources in this
+    tree is reported as stale (`profile_stale` in the roofline object)."""
     facts = {}
     pdir = os.path.join(ROOT, "profiles")
     if not os.path.isdir(pdir):
@@ -42,7 +60,8 @@ def profile_facts():
                     continue
                 kv = dict(tok.split("=", 1) for tok in line.split()[1:] if "=" in tok)
                 key = (kv.pop("kernel", ""), kv.pop("workload", ""))
-                ent = facts.setdefault(key, {"files": []})
+                ent = facts.setdefault(key, {"files": [], "src": set()})
+                ent["src"].add(kv.pop("src", None))
                 for k, v in kv.items():
                     ent[k] = float(v)
                 ent["files"].append("profiles/" + name)
@@ -63,6 +82,8 @@ def roofline_entry(kernel, workload, alg_bytes, kernel_ms, clock_hz, useful_valu
     f = (facts or {}).get((kernel, workload))
     if f:
         r["profile"] = sorted(set(f["files"]))
+        # counters taken from a library built from other sources than the ones in this tree describe another kernel
+        r["profile_stale"] = f["src"] != {kernel_source_hash()}
         if "traffic_bytes" in f:
             r["traffic"] = f["traffic_bytes"]
             r["physical_gbs"] = round(f["traffic_bytes"] / (kernel_ms * 1e-3) / 1e9, 1)
