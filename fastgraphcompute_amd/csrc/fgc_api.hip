@@ -200,7 +200,7 @@ extern "C" int fgc_binned_knn_prepare_ld_f32(const float *d_coords, int64_t n_ve
     rc = fgc_launch_prepare_tail(d_coords, ld_coords, order, skeys, (int)n_vert, n_coords, w.ldc, sc, d_direction, sdir,
                                  spp, fgc_knn_sp_half(n_coords), (float *)(ws + w.box_lo), (float *)(ws + w.box_hi),
                                  (float *)(ws + w.sbox_lo), (float *)(ws + w.sbox_hi), c.sub_bits * n_bin_dims,
-                                 (int)c.B, bb, s);
+                                 (int)c.B, bb, w.with_sp ? (unsigned *)(ws + w.mfstat) : nullptr, s);
     if (rc || !w.with_sp) return rc;
     return fgc_launch_mf_operands((const float *)(ws + w.sp), (const float *)(ws + w.box_lo),
                                   (const float *)(ws + w.box_hi), (int)n_vert, n_coords, w.ldc, (float *)(ws + w.grp),

@@ -915,9 +915,10 @@ __global__ __launch_bounds__(1024) void k_prepare_tail(const float *__restrict__
                                                        int sp_half, float *__restrict__ box_lo,
                                                        float *__restrict__ box_hi, float *__restrict__ sbox_lo,
                                                        float *__restrict__ sbox_hi, int key_shift, int n_bins_total,
-                                                       int *__restrict__ bb)
+                                                       int *__restrict__ bb, unsigned *__restrict__ zero2)
 {
     __shared__ float s_lo[16][16], s_hi[16][16];
+    if (zero2 && blockIdx.x == 0 && threadIdx.x < 2) zero2[threadIdx.x] = 0u;   // counters of the kernel that follows
     const int D = DT ? DT : D_rt;
     const int lane = fgc_lane(), wv = threadIdx.x >> 6;
     const int n_chunks = ldc / 64, n_super = (n_chunks + 63) / 64;
@@ -1035,14 +1036,14 @@ __global__ __launch_bounds__(1024) void k_prepare_tail(const float *__restrict__
 int fgc_launch_prepare_tail(const float *coords, int ld_in, const uint32_t *order, const uint32_t *skeys, int n, int D,
                             int ldc, float *sc, const int64_t *direction, unsigned char *sdir, float *sp, int sp_half,
                             float *box_lo, float *box_hi, float *sbox_lo, float *sbox_hi, int key_shift,
-                            int n_bins_total, int *bb, hipStream_t s)
+                            int n_bins_total, int *bb, unsigned *zero2, hipStream_t s)
 {
     // position n (the end of the last bin's run) must belong to a chunk some wavefront visits
     const int n_super = ((n + 1 + 63) / 64 + 63) / 64;
 #define FGC_TAIL(DT)                                                                                                    \
     hipLaunchKernelGGL(k_prepare_tail<DT>, dim3((unsigned)n_super), dim3(1024), 0, s, coords, ld_in, order, skeys, n, D, \
                        ldc, sc, direction, sdir, (float4 *)sp, sp_half, box_lo, box_hi, sbox_lo, sbox_hi, key_shift,   \
-                       n_bins_total, bb)
+                       n_bins_total, bb, zero2)
     switch (D) {
     case 2: FGC_TAIL(2); break;
     case 3: FGC_TAIL(3); break;

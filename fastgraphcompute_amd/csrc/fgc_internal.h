@@ -12,7 +12,7 @@ int fgc_launch_bin_keys(const float *d_coords, int n, int ld, int nbd, int sub_b
 int fgc_launch_prepare_tail(const float *coords, int ld_in, const uint32_t *order, const uint32_t *skeys, int n, int D,
                             int ldc, float *sc, const int64_t *direction, unsigned char *sdir, float *sp, int sp_half,
                             float *box_lo, float *box_hi, float *sbox_lo, float *sbox_hi, int key_shift,
-                            int n_bins_total, int *bb, hipStream_t s);
+                            int n_bins_total, int *bb, unsigned *zero2, hipStream_t s);
 bool fgc_sort_fused_fits(int64_t n);
 int fgc_keys_and_sort_fused(const float *coords, int n, int ld, int nbd, const int64_t *n_bins, int sub_bits,
                             int key_bits, const int64_t *rs, int n_rs, float *partial, float *geom, uint32_t *keys,

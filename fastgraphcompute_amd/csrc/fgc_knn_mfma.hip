@@ -77,37 +77,52 @@ using MfCollect = std::integral_constant<int, 2>;
 
 constexpr float MF_SHRINK16 = 1.0f - 0x1.08p-10f;    // 1 - 1.03 * 2^-10
 
-// Float16 operands of the candidates (see fgc_internal.h): one wavefront per chunk, lane = point.
-__global__ __launch_bounds__(256) void k_mf_operands(const float4 *__restrict__ sp4, const float *__restrict__ box_lo,
-                                                     const float *__restrict__ box_hi, int n, int D, int DH, int ldc,
-                                                     int n_chunks, float *__restrict__ grp, uint4 *__restrict__ spa,
-                                                     unsigned *__restrict__ mfstat)
+// Float16 operands of the candidates (see fgc_internal.h): one block per group of chunks, one wavefront per chunk,
+// lane = point.
+__global__ __launch_bounds__(64 * FGC_MF_GROUP_CHUNKS) void k_mf_operands(
+    const float4 *__restrict__ sp4, const float *__restrict__ box_lo, const float *__restrict__ box_hi, int n, int D, int DH,
+    int ldc, int n_chunks, float *__restrict__ grp, uint4 *__restrict__ spa, unsigned *__restrict__ mfstat)
 {
+    __shared__ unsigned s_wide, s_chunks;
     const int lane = fgc_lane();
-    const int c = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
-    if (c >= n_chunks) return;
-    const int g = c / FGC_MF_GROUP_CHUNKS;
+    const int g = blockIdx.x;
+    const int c = g * FGC_MF_GROUP_CHUNKS + (int)(threadIdx.x >> 6);
+    if (threadIdx.x == 0) { s_wide = 0u; s_chunks = 0u; }
+    __syncthreads();
     // bounding box of the group, coordinate d in lane d
     float lo = INFINITY, hi = -INFINITY;
-    if (lane < D)
-        for (int cc = g * FGC_MF_GROUP_CHUNKS; cc < min((g + 1) * FGC_MF_GROUP_CHUNKS, n_chunks); cc++) {
-            lo = fminf(lo, box_lo[(size_t)lane * n_chunks + cc]);
-            hi = fmaxf(hi, box_hi[(size_t)lane * n_chunks + cc]);
+    if (lane < D) {
+        float l[FGC_MF_GROUP_CHUNKS], h[FGC_MF_GROUP_CHUNKS];
+#pragma unroll
+        for (int k = 0; k < FGC_MF_GROUP_CHUNKS; k++) {
+            const int cc = g * FGC_MF_GROUP_CHUNKS + k;
+            l[k] = cc < n_chunks ? box_lo[(size_t)lane * n_chunks + cc] : INFINITY;
+            h[k] = cc < n_chunks ? box_hi[(size_t)lane * n_chunks + cc] : -INFINITY;
         }
+#pragma unroll
+        for (int k = 0; k < FGC_MF_GROUP_CHUNKS; k++) { lo = fminf(lo, l[k]); hi = fmaxf(hi, h[k]); }
+    }
     // How wide is the group against its own chunks?  Where a group of 1024 points spans several clusters while its
     // chunks of 64 sit inside one, the float16 screening error (proportional to the group's squared radius) exceeds
-    // the neighbour distances and the matrix-core search could only hand its queries on: counted here, decided there.
-    {
+    // the neighbour distances and the matrix-core search could only hand its queries on: counted here (one pair of
+    // adds per group), decided there.
+    if (c < n_chunks) {
         const float clo = lane < D ? box_lo[(size_t)lane * n_chunks + c] : 0.f;
         const float chi = lane < D ? box_hi[(size_t)lane * n_chunks + c] : 0.f;
         const float ch = (lane < D && fabsf(clo) < INFINITY && fabsf(chi) < INFINITY && chi >= clo) ? 0.5f * chi - 0.5f * clo : 0.f;
         const float gh = (lane < D && fabsf(lo) < INFINITY && fabsf(hi) < INFINITY && hi >= lo) ? 0.5f * hi - 0.5f * lo : 0.f;
         const float rc2 = fgc_wave_sum(ch * ch), rg2 = fgc_wave_sum(gh * gh);
         if (lane == 0 && c * 64 < n) {
-            atomicAdd(&mfstat[0], 1u);
-            if (rg2 > 24.f * rc2) atomicAdd(&mfstat[1], 1u);
+            atomicAdd(&s_chunks, 1u);
+            if (rg2 > 24.f * rc2) atomicAdd(&s_wide, 1u);
         }
     }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        if (s_chunks) atomicAdd(&mfstat[0], s_chunks);
+        if (s_wide) atomicAdd(&mfstat[1], s_wide);
+    }
+    if (c >= n_chunks) return;
     float ctr = 0.5f * lo + 0.5f * hi, half = 0.5f * hi - 0.5f * lo;
     if (lane >= D) { ctr = 0.f; half = 0.f; }
     else if (!(fabsf(lo) < INFINITY && fabsf(hi) < INFINITY)) { ctr = 0.f; half = lo > hi ? 0.f : INFINITY; }   // lo > hi: no finite point
@@ -162,11 +177,11 @@ __global__ __launch_bounds__(256) void k_mf_operands(const float4 *__restrict__ 
 int fgc_launch_mf_operands(const float *sp, const float *box_lo, const float *box_hi, int n, int D, int ldc, float *grp,
                            void *spa, unsigned *mfstat, hipStream_t s)
 {
+    // (mfstat[0..1] start at zero: cleared by the kernel that wrote the boxes, fgc_launch_prepare_tail)
     const int n_chunks = ldc / 64;
-    int rc = fgc_fill_u32(mfstat, 0u, 2, s);
-    if (rc) return rc;
-    hipLaunchKernelGGL(k_mf_operands, dim3((unsigned)fgc_cdiv(n_chunks, 4)), dim3(256), 0, s, (const float4 *)sp, box_lo,
-                       box_hi, n, D, fgc_knn_sp_half(D), ldc, n_chunks, grp, (uint4 *)spa, mfstat);
+    hipLaunchKernelGGL(k_mf_operands, dim3((unsigned)fgc_cdiv(n_chunks, FGC_MF_GROUP_CHUNKS)), dim3(64 * FGC_MF_GROUP_CHUNKS),
+                       0, s, (const float4 *)sp, box_lo, box_hi, n, D, fgc_knn_sp_half(D), ldc, n_chunks, grp, (uint4 *)spa,
+                       mfstat);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
