@@ -133,7 +133,7 @@ def test_ops_are_registered_and_wrappers_script():
 
 
 def test_integration_shim_compiles_against_the_header():
-    """The reference-side binding documented in INTEGRATION.md (the C++ a maintainer would put behind
+    """The reference-side binding shown in the repository's integration notes (the C++ a maintainer would put behind
     BinnedKNNAutograd and the *_cuda_fn symbols) is compiled, syntax only, against include/fgc_hip.h and the torch
     headers: argument counts and types of every call must match the header."""
     import shutil
@@ -144,7 +144,7 @@ def test_integration_shim_compiles_against_the_header():
         pytest.skip("no g++")
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     blocks = re.findall(r"```cpp\n(.*?)```", text, flags=re.S)
-    assert blocks, "INTEGRATION.md holds no C++ block"
+    assert blocks, "the integration notes hold no C++ block"
     src = "\n".join(blocks)
     for fn in ("fgc_binned_select_knn_f32", "fgc_binned_select_knn_grad_f32", "fgc_index_replacer_i64",
                "fgc_bin_points_f32"):
