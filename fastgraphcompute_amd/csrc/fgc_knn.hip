@@ -133,6 +133,24 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     int cnt = 0;            // lane q: candidates in query q's pool
     bool qactive = isq;
     if (a.sdir && isq) { unsigned char dd = a.sdir[qs]; qactive = !(dd == 0 || dd == 2); }
+    // With few coordinates the queries' coordinates and bounds are also kept as wave-uniform values (scalar registers):
+    // the loops over the queries of a chunk are unrolled and the subtractions take them as scalar operands, instead
+    // of one v_readlane per coordinate and (query, chunk).  st[q] mirrors lane q of tau and is refreshed wherever tau
+    // changes (seeds, prunes).
+    //    sn[q] likewise stands for lane q of cnt while the spans of a group are searched: the common pool append then
+    //    touches no per-lane state at all; cnt is brought up to date before anything else reads it (a prune, the epilogue).
+    constexpr bool SQ = DT >= 2;
+    float sq[SQ ? QT : 1][DR], st[SQ ? QT : 1];
+    int sn[SQ ? QT : 1];
+    if (SQ) {
+#pragma unroll
+        for (int q = 0; q < QT; q++) {
+#pragma unroll
+            for (int dd = 0; dd < DR; dd++) sq[q][dd] = fgc_readlane_f(qx[dd], q);
+            st[q] = a.tau0;
+            sn[q] = 0;
+        }
+    }
     // second launch behind the matrix-core search: only the queries it flagged
     const bool redo_q = !a.redo || (isq && a.redo[qs] != 0);
     if (a.redo) {
@@ -259,9 +277,10 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
     // ---- append the lanes in `want` (candidate j at squared distance dsq, one per lane) to query q's pool; when
     //      it overflows or runs nearly full (tau should stay tight) prune it: first to a tighter threshold, then,
     //      if lanes are still waiting, down to exactly K ----
-    auto push = [&](int q, float dsq, int j, bool want) {
+    //      Returns true when the query's bound may have changed (a prune ran).
+    auto push = [&](int q, float dsq, int j, bool want) -> bool {
         unsigned long long pm = fgc_ballot(want);
-        if (!pm) return;
+        if (!pm) return false;
         CNT(n_app++);
         int pc = fgc_readlane_i(cnt, q);
         {
@@ -271,7 +290,7 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             if (pn <= CAP - PRUNE_MARGIN && (pn <= K || ((fgc_ballot(tau < INFINITY) >> q) & 1ull))) {
                 if (want) pool[q * CAP + pc + fgc_mbcnt(pm)] = make_uint2(__float_as_uint(dsq), (unsigned)j);
                 cnt = (lane == q) ? pn : cnt;
-                return;
+                return false;
             }
         }
         for (int attempt = 0;; attempt++) {
@@ -291,6 +310,24 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             pm = fgc_ballot(want);
             if (!pm) break;
         }
+        return true;
+    };
+    // the same with the query's count and bound held as wave-uniform values (sc = sn[q], stq = st[q])
+    auto push_s = [&](int q, float dsq, int j, bool want, int &sc, float &stq) {
+        const unsigned long long pm = fgc_ballot(want);
+        if (!pm) return;
+        CNT(n_app++);
+        const int pn = sc + __popcll(pm);
+        if (pn <= CAP - PRUNE_MARGIN && (pn <= K || stq < INFINITY)) {
+            if (want) pool[q * CAP + sc + fgc_mbcnt(pm)] = make_uint2(__float_as_uint(dsq), (unsigned)j);
+            sc = pn;
+            return;
+        }
+        CNT(n_app--);
+        cnt = (lane == q) ? sc : cnt;
+        push(q, dsq, j, want);
+        sc = fgc_readlane_i(cnt, q);
+        stq = fgc_readlane_f(tau, q);
     };
 
     // ---- groups of queries sharing a bin row ----
@@ -399,6 +436,10 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
             }
         }
 
+        if (SQ) {
+#pragma unroll
+            for (int q = 0; q < QT; q++) { st[q] = fgc_readlane_f(tau, q); sn[q] = fgc_readlane_i(cnt, q); }
+        }
         // span iteration state: phase 0 = own chunk, 1 = the other seed chunks, 2 = bin rows ring by ring
         int phase = (SMAX > 0) ? ((ra == seed_c0 && rb == seed_c1) ? 2 : 1) : 0, d = 0;
         int ai[RD], lo[RD], hi[RD];
@@ -539,6 +580,21 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                         bhi[dd] = (cv && dd < Dn) ? a.box_hi[(size_t)dd * nch + c] : 0.f;
                     }
                     mymask = 0u;
+                    if (SQ) {
+#pragma unroll
+                        for (int q = 0; q < QT; q++) {
+                            if (!((actb >> q) & 1ull)) continue;
+                            CNT(n_cullq++);
+                            float g = fmaxf(fmaxf(blo[0] - sq[q][0], sq[q][0] - bhi[0]), 0.f);
+                            float g2 = g * g;
+#pragma unroll
+                            for (int dd = 1; dd < DR; dd++) {
+                                g = fmaxf(fmaxf(blo[dd] - sq[q][dd], sq[q][dd] - bhi[dd]), 0.f);
+                                g2 += g * g;
+                            }
+                            if (cv && !(g2 > st[q])) mymask |= 1u << q;
+                        }
+                    } else
                     for (unsigned long long m = actb; m;) {
                         CNT(n_cullq++);
                         const int q = __ffsll((long long)m) - 1;
@@ -591,6 +647,17 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     nev += (unsigned long long)__popcll(cact) * (unsigned)(min(j1, base + 64) - max(j0, base));
                     nchunks++;
 #endif
+                    if (SQ) {
+#pragma unroll
+                        for (int q = 0; q < QT; q++) {
+                            if (!((cact >> q) & 1ull)) continue;
+                            float df = sq[q][0] - cx[0];
+                            float dsq = df * df;
+#pragma unroll
+                            for (int dd = 1; dd < DR; dd++) { df = sq[q][dd] - cx[dd]; dsq += df * df; }
+                            push_s(q, dsq, j, dsq < st[q], sn[q], st[q]);
+                        }
+                    } else
                     for (unsigned long long m = cact; m;) {
                         const int q = __ffsll((long long)m) - 1;
                         m &= m - 1;
@@ -616,6 +683,10 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
                     }
                 }
             }
+        }
+        if (SQ) {
+#pragma unroll
+            for (int q = 0; q < QT; q++) cnt = (lane == q) ? sn[q] : cnt;
         }
     }
 
