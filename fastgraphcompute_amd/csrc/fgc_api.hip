@@ -243,8 +243,9 @@ int knn_search(float tau0, int32_t *d_nbr_sorted, int64_t n_vert, int32_t n_coor
     a.mfstat = c.w.with_sp ? (const unsigned *)(ws + c.w.mfstat) : nullptr;
     a.redo = nullptr;
     // Many coordinates and events that the bounding boxes cannot thin out: the matrix-core search.  Measured on
-    // uniform and clustered points with 1 000 to 65 000 points per event: it wins up to about 1024 * 4^(D - 5)
-    // points per event (twice that from K = 64 on), where the size is the one a typical point sees, sum n_e^2 / n.
+    // uniform and clustered points with 1 000 to 65 000 points per event: it wins up to about 1536 * 3^(D - 5)
+    // points per event (half as many again from K = 64 on), where the size is the one a typical point sees,
+    // sum n_e^2 / n.
     // It stores candidates as 16-bit positions inside their event, so no event may exceed 65535 points.  A search
     // with a radius bound keeps the vector search, which culls by the bound from the first bin row on.
     int64_t largest_event = 0;
@@ -255,9 +256,9 @@ int knn_search(float tau0, int32_t *d_nbr_sorted, int64_t n_vert, int32_t n_coor
         sum_sq += (double)ne * (double)ne;
     }
     const double typical_event = n_vert > 0 ? sum_sq / (double)n_vert : 0.0;
-    double limit = 1024.0;
-    for (int d = 5; d < n_coords; d++) limit *= 4.0;
-    if (K >= 64) limit *= 2.0;
+    double limit = 1536.0;
+    for (int d = 5; d < n_coords; d++) limit *= 3.0;
+    if (K >= 64) limit *= 1.5;
     limit = std::min(limit, 32768.0);
     const bool force = (tf_compat & FGC_KNN_FORCE_MATRIX) != 0;
     if (a.sp && !(tf_compat & FGC_KNN_NO_MATRIX) && !(tau0 < INFINITY) && largest_event <= 65535 &&
