@@ -351,7 +351,8 @@ __device__ __forceinline__ float fgc_wave_reduce16(const float (&v)[16], int lan
 // the coordinates of a target in adjacent lanes and neighbouring targets in neighbouring lanes, which for the
 // window part are neighbouring addresses; k_unsort_grad moves the rows to the original order.
 // PACK (D <= 3): a table entry is one float4 (x, y, z, tag) - value and tag in one 16-byte LDS access.
-template <bool PACK>
+// D4T: float4 groups per point where the kernel is built for exactly that many (1 or 2: up to 8 coordinates), 0 = any.
+template <bool PACK, int D4T>
 __global__ __launch_bounds__(64) void k_knn_grad_sorted(const float *__restrict__ gd, const int *__restrict__ nbr,
                                                         const float4 *__restrict__ xs,
                                                         const uint32_t *__restrict__ order, float *__restrict__ gxs,
@@ -359,7 +360,7 @@ __global__ __launch_bounds__(64) void k_knn_grad_sorted(const float *__restrict_
 {
     extern __shared__ __align__(16) unsigned char s_raw[];
     const int lane = fgc_lane();
-    const int D4 = PACK ? 1 : (D + 3) >> 2;
+    const int D4 = PACK ? 1 : (D4T ? D4T : (D + 3) >> 2);
     const int ld = D4 * 4;                     // floats per row of xs and gxs
     float4 *vals = (float4 *)s_raw;            // [H][D4]
     unsigned *tags = PACK ? (unsigned *)vals + 3 : (unsigned *)(s_raw + (size_t)H * 16 * D4);
@@ -578,15 +579,20 @@ extern "C" int fgc_binned_select_knn_grad_sorted_ld_f32(const float *d_grad_dist
     FGC_LAUNCH_CHECK();
     if (n_coords <= 3) {
         const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GSW);
-        hipLaunchKernelGGL((k_knn_grad_sorted<true>), dim3(blocks), dim3(64), (size_t)GSH * (16 + sizeof(GRAD_OWNER_T)), s, d_grad_distsq,
+        hipLaunchKernelGGL((k_knn_grad_sorted<true, 1>), dim3(blocks), dim3(64), (size_t)GSH * (16 + sizeof(GRAD_OWNER_T)), s, d_grad_distsq,
                            d_nbr_sorted, (const float4 *)xs, (const uint32_t *)d_order, gxs, n_vert, (int)K,
                            (int)n_coords, GSH, d_status);
     } else {
         const int H = grad_table_size(n_coords);
         const unsigned blocks = (unsigned)fgc_cdiv(n_vert, GW);
-        hipLaunchKernelGGL((k_knn_grad_sorted<false>), dim3(blocks), dim3(64), (size_t)H * (8 + 16 * (size_t)D4), s,
-                           d_grad_distsq, d_nbr_sorted, (const float4 *)xs, (const uint32_t *)d_order, gxs, n_vert,
-                           (int)K, (int)n_coords, H, d_status);
+#define FGC_GRAD_WIDE(D4T)                                                                                              \
+    hipLaunchKernelGGL((k_knn_grad_sorted<false, D4T>), dim3(blocks), dim3(64), (size_t)H * (8 + 16 * (size_t)D4), s,   \
+                       d_grad_distsq, d_nbr_sorted, (const float4 *)xs, (const uint32_t *)d_order, gxs, n_vert, (int)K, \
+                       (int)n_coords, H, d_status)
+        if (D4 == 1) FGC_GRAD_WIDE(1);
+        else if (D4 == 2) FGC_GRAD_WIDE(2);
+        else FGC_GRAD_WIDE(0);
+#undef FGC_GRAD_WIDE
     }
     FGC_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_unsort_grad, dim3((unsigned)fgc_cdiv(n_vert * D4, 256)), dim3(256), 0, s, (const float4 *)gxs,
