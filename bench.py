@@ -242,10 +242,10 @@ def main():
     # those are its distance evaluations; the screened pairs are reported separately)
     n_exact = collected if matrix else c_eval
     bytes_alg = 4.0 * D * n_exact + 4.0 * D * n + 12.0 * K * n
-    # VALU wavefront instructions that are distance arithmetic: per 64 evaluations D subtractions, D
-    # multiplications, D - 1 additions, the compare, and the D + 1 broadcasts of the query and its bound
+    # VALU wavefront instructions that are distance arithmetic: per 64 evaluations D subtractions (the query's
+    # coordinates are scalar operands), D multiplications, D - 1 additions and the compare
     roofline = roofline_entry("k_knn_mf" if matrix else "k_knn", w["name"], bytes_alg, t_knn, clock_hz,
-                              None if matrix else (c_eval / 64.0) * (4 * D + 1), facts)
+                              None if matrix else (c_eval / 64.0) * (3 * D), facts)
     if matrix:
         # one v_mfma_f32_32x32x16_f16 per 32 x 32 pairs: 32 flops per evaluated pair, against the dense float16 peak
         roofline["screened_pairs"] = c_eval
