@@ -53,8 +53,14 @@
 #undef FGC_KNN_COUNTERS        // the debug counters exist in the statistics build only
 #endif
 
-#ifndef QT
-#define QT 6           // queries per wavefront (6 x 128 pool slots x 8 B = 6 KB of LDS at K = 64: 26 wavefronts per CU)
+#ifndef QT_DEFAULT
+#define QT_DEFAULT 6   // queries per wavefront (6 x 128 pool slots x 8 B = 6 KB of LDS at K = 64: 26 wavefronts per CU)
+#endif
+#ifndef QT_SMALL
+#define QT_SMALL 3     // for inputs too small to fill the GPU with wavefronts of 6 queries: twice the wavefronts, each with
+#endif                 // half the serial work (search of 10 000 points, D = 3, K = 40: 45 -> 33 us; 40 000: 88 -> 82; 80 000: 142 -> 147)
+#ifndef KNN_SMALL_N
+#define KNN_SMALL_N 49152
 #endif
 #ifndef POOL_EXTRA
 #define POOL_EXTRA 48  // pool slots beyond K (rounded up to 16); LDS per wavefront = QT * pool slots * 8 B
@@ -77,8 +83,8 @@
 template <int NSEG> struct KnnCfg { static constexpr int WPB = 1; };
 
 // DT: coordinates per point held in registers (0 = any number, read from memory)
-// NSEG: ceil(K / 64);  RD: bin-row dimensions (binned dimensions - 1, padded)
-template <int DT, int NSEG, int RD>
+// NSEG: ceil(K / 64);  RD: bin-row dimensions (binned dimensions - 1, padded);  QT: queries per wavefront
+template <int DT, int NSEG, int RD, int QT>
 __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 {
     constexpr int PS = NSEG + 1;          // pool segments (lanes x PS cover the pool)
@@ -793,13 +799,13 @@ __global__ __launch_bounds__(KnnCfg<NSEG>::WPB * 64) void k_knn(KnnArgs a)
 #endif
 }
 
-template <int DT, int NSEG, int RD> static int launch_knn_t(const KnnArgs &a, hipStream_t s)
+template <int DT, int NSEG, int RD, int QT = QT_DEFAULT> static int launch_knn_t(const KnnArgs &a, hipStream_t s)
 {
     constexpr int WPB = KnnCfg<NSEG>::WPB;
     const int tiles = (int)fgc_cdiv(a.n, QT);
     const int blocks = (int)fgc_cdiv(tiles, WPB);
     const size_t lds = (size_t)WPB * 2 * QT * a.pool_cap * sizeof(float);
-    hipLaunchKernelGGL((k_knn<DT, NSEG, RD>), dim3(blocks), dim3(WPB * 64), lds, s, a);
+    hipLaunchKernelGGL((k_knn<DT, NSEG, RD, QT>), dim3(blocks), dim3(WPB * 64), lds, s, a);
     FGC_LAUNCH_CHECK();
     return FGC_OK;
 }
@@ -807,13 +813,22 @@ template <int DT, int NSEG, int RD> static int launch_knn_t(const KnnArgs &a, hi
 // Kernels with the coordinates in registers are built for the combinations of coordinate count and binned dimensions
 // that the two grid rules produce (the library's own grid bins min(D, 5) dimensions, the reference's rule 3 - or 2
 // for D = 2); any other combination (a caller's max_bin_dims) runs the variant that reads coordinates from memory.
+// up to four coordinates and 64 neighbours: small inputs get wavefronts of QT_SMALL queries
+template <int DT, int NSEG, int RD> static int launch_knn_q(const KnnArgs &a, hipStream_t s)
+{
+    if constexpr (NSEG == 1) {
+        if (a.n <= KNN_SMALL_N) return launch_knn_t<DT, NSEG, RD, QT_SMALL>(a, s);
+    }
+    return launch_knn_t<DT, NSEG, RD>(a, s);
+}
+
 template <int NSEG, int RD> static int launch_knn_d(const KnnArgs &a, hipStream_t s)
 {
     constexpr bool wide = RD == 2 || RD == 4;      // 3 or 5 binned dimensions
     switch (a.D) {
-    case 2: if constexpr (RD == 1) return launch_knn_t<2, NSEG, RD>(a, s); break;
-    case 3: if constexpr (RD == 2) return launch_knn_t<3, NSEG, RD>(a, s); break;
-    case 4: if constexpr (RD == 2 || RD == 3) return launch_knn_t<4, NSEG, RD>(a, s); break;
+    case 2: if constexpr (RD == 1) return launch_knn_q<2, NSEG, RD>(a, s); break;
+    case 3: if constexpr (RD == 2) return launch_knn_q<3, NSEG, RD>(a, s); break;
+    case 4: if constexpr (RD == 2 || RD == 3) return launch_knn_q<4, NSEG, RD>(a, s); break;
     case 5: if constexpr (wide) return launch_knn_t<5, NSEG, RD>(a, s); break;
     case 6: if constexpr (wide) return launch_knn_t<6, NSEG, RD>(a, s); break;
     case 7: if constexpr (wide) return launch_knn_t<7, NSEG, RD>(a, s); break;
