@@ -104,7 +104,31 @@ def require_device(*tensors):
 
 
 def stream_ptr():
+    """The current HIP stream of the current device as a void pointer."""
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None:         # (what torch.cuda.current_stream().cuda_stream returns, without building a Stream object)
+        return ctypes.c_void_p(raw(torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class on_device:
+    """`with on_device(dev):` makes `dev` the current device like torch.cuda.device(dev), but does nothing at all when it
+    already is (the usual case, and a few microseconds per call on the small-input path)."""
+    __slots__ = ("ctx",)
+
+    def __init__(self, dev):
+        idx = dev.index if isinstance(dev, torch.device) else int(dev)
+        self.ctx = None if (idx is None or idx == torch.cuda.current_device()) else torch.cuda.device(idx)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+        return self
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        return False
 
 
 def ptr(t):

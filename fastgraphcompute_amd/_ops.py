@@ -81,7 +81,7 @@ def _bin_by_coordinates_impl(coordinates: torch.Tensor, row_splits: torch.Tensor
     ws_bytes = L.fgc_bin_geometry_workspace_bytes(n)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     nb_arr = _lib.host_i64(nb_host if nb_host is not None else [1] * d)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         st = _lib.stream_ptr()
         _lib.check(L.fgc_bin_geometry_f32(_lib.ptr(coords), n, d, d, 1 if have_bw else 0, nb_arr,
                                           1 if nb_host is not None else 0, bw_host, 1 if pre_normalized else 0,
@@ -158,7 +158,7 @@ def knn_grad(grad_distsq: torch.Tensor, idx: torch.Tensor, coords: torch.Tensor,
         order = order.to(device=x.device, dtype=torch.int32).contiguous()
         if order.numel() != n:
             raise ValueError("order must hold one entry per point")
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         _lib.check(L.fgc_binned_select_knn_grad_f32(_lib.ptr(g), _lib.ptr(ii), _lib.ptr(x), _lib.ptr(out), n, K, D,
                                                     _lib.ptr(order), _lib.ptr(status), _lib.stream_ptr()))
     _raise_on_bad_index(status, "binned_select_knn_grad")
@@ -210,7 +210,7 @@ def knn_grad_sorted(grad_distsq: torch.Tensor, nbr_sorted: torch.Tensor, coords:
         out = torch.empty((n, D), dtype=torch.float32, device=x.device)
     ws_bytes = L.fgc_binned_select_knn_grad_sorted_workspace_bytes(n, D)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         # no status word: the rows come from the library's own search, and nothing on this path reads it
         _lib.check(L.fgc_binned_select_knn_grad_sorted_ld_f32(
             _lib.ptr(g), _lib.ptr(nbr_sorted), _lib.ptr(x), ld, _lib.ptr(order), _lib.ptr(out), out.stride(0), n, K, D,
@@ -306,7 +306,7 @@ def _knn_forward(coords: torch.Tensor, D: int, row_splits, K: int, direction, n_
     rs_dev = rs_dev.contiguous()
     idx = torch.empty((n, K), dtype=torch.int64, device=dev)
     dist = torch.empty((n, K), dtype=torch.float32, device=dev)
-    order = torch.empty(0, dtype=torch.int32, device=dev)
+    order = None
     nbr_sorted = None
     if n > 0:
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
@@ -315,7 +315,7 @@ def _knn_forward(coords: torch.Tensor, D: int, row_splits, K: int, direction, n_
         dirt = None
         if direction is not None and direction.numel() > 0:
             dirt = direction.to(device=dev, dtype=torch.int64).contiguous()
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             st = _lib.stream_ptr()
             # prepare and search are enqueued separately so that the input checks (status word, written by
             # the prepare stage) can be read back while the search is already queued behind them: the host
@@ -359,6 +359,8 @@ def _knn_forward(coords: torch.Tensor, D: int, row_splits, K: int, direction, n_
                                   n_bins=nb, n_vert=n, K=K, n_coords=D)
     if nbr_sorted is None:
         nbr_sorted = torch.empty((0, K), dtype=torch.int32, device=dev)
+    if order is None:
+        order = torch.empty(0, dtype=torch.int32, device=dev)
     return idx, dist, nbr_sorted, order
 
 
@@ -421,7 +423,7 @@ def _index_replacer_impl(to_be_replaced: torch.Tensor, replacements: torch.Tenso
     src = to_be_replaced.contiguous()
     rep = replacements.contiguous()
     out = torch.empty_like(src)
-    with torch.cuda.device(src.device):
+    with _lib.on_device(src.device):
         _lib.check(L.fgc_index_replacer_i64(_lib.ptr(src), _lib.ptr(rep), _lib.ptr(out), src.numel(), rep.numel(),
                                             _lib.stream_ptr()))
     return out
@@ -438,7 +440,7 @@ class _SelectWithDefault(torch.autograd.Function):
         V, K = ii.shape
         rows, F = ff.shape
         out = torch.empty((V, K, F), dtype=ff.dtype, device=ff.device)
-        with torch.cuda.device(ff.device):
+        with _lib.on_device(ff.device):
             if ff.dtype == torch.float32:
                 _lib.check(L.fgc_select_with_default_f32(_lib.ptr(ii), _lib.ptr(ff), _lib.ptr(out), V, K, F, rows,
                                                          float(default_value), _lib.stream_ptr()))
@@ -488,7 +490,7 @@ class _GravNetAggregate(torch.autograd.Function):
         fmax = torch.empty((n, P), dtype=torch.float32, device=f.device)
         argmax = torch.empty((n, P), dtype=torch.int32, device=f.device)
         status = torch.zeros(4, dtype=torch.int32, device=f.device)
-        with torch.cuda.device(f.device):
+        with _lib.on_device(f.device):
             _lib.check(L.fgc_gravnet_aggregate_fwd_ld_f32(_lib.ptr(ii), _lib.ptr(d), _lib.ptr(f), P, f.shape[0],
                                                           _lib.ptr(fmean), _lib.ptr(fmax), P, _lib.ptr(argmax), n, K, P,
                                                           _lib.ptr(status), _lib.stream_ptr()))
@@ -511,7 +513,7 @@ class _GravNetAggregate(torch.autograd.Function):
             else g_max.to(torch.float32).contiguous()
         g_feat = torch.zeros_like(f)
         g_dist = torch.empty_like(d)
-        with torch.cuda.device(f.device):
+        with _lib.on_device(f.device):
             _lib.check(L.fgc_gravnet_aggregate_bwd_f32(_lib.ptr(ii), _lib.ptr(d), _lib.ptr(f), _lib.ptr(argmax),
                                                        _lib.ptr(g_mean), _lib.ptr(g_max), _lib.ptr(g_feat),
                                                        _lib.ptr(g_dist), n, K, P, _lib.stream_ptr()))
@@ -544,7 +546,7 @@ class _GravNetLayerCore(torch.autograd.Function):
         agg = torch.empty((n, 2 * P), dtype=torch.float32, device=dev)
         argmax = torch.empty((n, P), dtype=torch.int32, device=dev)
         if n > 0:
-            with torch.cuda.device(dev):
+            with _lib.on_device(dev):
                 _lib.check(L.fgc_gravnet_aggregate_fwd_ld_f32(
                     _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(feat), P, n, _lib.ptr(agg),
                     ctypes.c_void_p(agg.data_ptr() + 4 * P), 2 * P, _lib.ptr(argmax), n, K, P, None,
@@ -566,7 +568,7 @@ class _GravNetLayerCore(torch.autograd.Function):
                 g_agg = g_agg.to(torch.float32).contiguous()
             g_feat = torch.zeros_like(feat)
             g_dsq = torch.empty_like(dist)
-            with torch.cuda.device(feat.device):
+            with _lib.on_device(feat.device):
                 if config.tile_aggregation_backward and nbr_sorted.shape[0] == n and \
                         L.fgc_gravnet_aggregate_bwd_sorted_supported(n, K, P, P, P):
                     # rows that are neighbours in the search's sorted order share their targets: combined on chip
@@ -663,7 +665,7 @@ def _oc_objects(asso: torch.Tensor, row_splits: torch.Tensor, filter_negative: b
     objects_per_split = torch.empty(n_rs - 1, dtype=torch.int64, device=dev)
     wide = 0
     while True:
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             _lib.check(L.fgc_oc_helper_objects_i64(_lib.ptr(a), n, _lib.ptr(rs), n_rs, int(filter_negative), wide,
                                                    _lib.ptr(max_per_split), _lib.ptr(objects_per_split),
                                                    _lib.ptr(summary), _lib.ptr(ws), ws_bytes, _lib.stream_ptr()))
@@ -690,7 +692,7 @@ def _oc_helper_matrices_impl(truth_idxs: torch.Tensor, row_splits: torch.Tensor,
     M = torch.empty((n_unique, n_maxuq), dtype=torch.int64, device=dev)
     # without M_not the reference's device op hands back an empty [0, 0] tensor (oc_helper_cuda_kernel.cu:171-176)
     M_not = torch.empty((n_unique, n_maxrs) if calc_m_not else (0, 0), dtype=torch.int64, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(L.fgc_oc_helper_fill_i64(a.numel(), _lib.ptr(rs), rs.numel(), n_unique, n_maxuq, n_maxrs, None, None,
                                             _lib.ptr(summary), _lib.ptr(M), _lib.ptr(M_not) if calc_m_not else None,
                                             None, None, None, _lib.ptr(ws), ws_bytes, _lib.stream_ptr()))
@@ -724,7 +726,7 @@ def _oc_helper_cuda_impl(asso_idx: torch.Tensor, unique_idx: torch.Tensor, uniqu
     M = torch.empty((n_rows, n_maxuq), dtype=torch.int64, device=dev)
     M_not = torch.empty((n_rows, n_maxrs) if calc_m_not else (0, 0), dtype=torch.int64, device=dev)
     status = torch.zeros(4, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(L.fgc_oc_helper_fill_i64(a.numel(), _lib.ptr(rsd), rsd.numel(), n_rows, n_maxuq, n_maxrs,
                                             _lib.ptr(unique_idx), _lib.ptr(unique_rs_asso), _lib.ptr(summary),
                                             _lib.ptr(M), _lib.ptr(M_not) if calc_m_not else None, None, None,
@@ -779,7 +781,7 @@ def _select_knn_impl(coords: torch.Tensor, row_splits: torch.Tensor, mask: torch
     ws_bytes = L.fgc_binned_select_knn_workspace_bytes(n, D, nbd, nb_arr, n_rs, K)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     status = torch.zeros(4, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(L.fgc_select_knn_f32(_lib.ptr(x), n, D, _lib.ptr(rs_dev), rs_arr, n_rs, K, float(max_radius), nbd,
                                         nb_arr, _lib.ptr(idx), _lib.ptr(dist), _lib.ptr(status), _lib.ptr(ws),
                                         ws_bytes, _lib.stream_ptr()))
@@ -801,7 +803,7 @@ def linear_wgrad(grad_out: torch.Tensor, x: torch.Tensor, with_bias: bool = True
     gb = torch.empty(O, dtype=torch.float32, device=g.device) if with_bias else None
     ws_bytes = L.fgc_linear_wgrad_workspace_bytes(n, O, I)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=g.device)
-    with torch.cuda.device(g.device):
+    with _lib.on_device(g.device):
         _lib.check(L.fgc_linear_wgrad_f32(_lib.ptr(g), _lib.ptr(xx), n, O, I, _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(ws),
                                           ws_bytes, _lib.stream_ptr()))
     return gw, gb
