@@ -7,11 +7,12 @@
 //
 // Candidates are streamed one chunk at a time, one candidate per lane, with
 // coalesced loads from the structure-of-arrays coordinate copy; the wavefront
-// then walks over the queries that still need the chunk (query coordinates
-// broadcast from the owning lane), so a loaded candidate is reused by up to QT
+// then walks over the queries that still need the chunk (the queries' coordinates,
+// bounds and pool counts are held as wave-uniform values in scalar registers, the
+// walk is unrolled over them), so a loaded candidate is reused by up to QT
 // queries.  Each query owns an unsorted candidate pool in LDS (K kept + room for
 // one more chunk); tau_q, an upper bound of the query's K-th distance, lives in
-// lane q of a register.  Lanes that beat tau append themselves to the pool
+// lane q of a register (and in a scalar copy).  Lanes that beat tau append themselves to the pool
 // (ballot + prefix count, no sorting); when the pool runs full it is pruned: a
 // bisection on the distance threshold, counted with wave ballots over the pool
 // held one slot per lane, finds a tighter tau and the survivors are compacted.
