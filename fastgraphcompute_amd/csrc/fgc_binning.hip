@@ -1016,7 +1016,7 @@ __global__ __launch_bounds__(1024) void k_prepare_tail(const float *__restrict__
         s_lo[wv][lane] = lo; s_hi[wv][lane] = hi;
     }
     __syncthreads();
-    if (g < n_super && threadIdx.x < min(D, 16)) {
+    if (g < n_super && (int)threadIdx.x < min(D, 16)) {
         float lo = INFINITY, hi = -INFINITY;
         for (int w = 0; w < 16; w++) { lo = fminf(lo, s_lo[w][threadIdx.x]); hi = fmaxf(hi, s_hi[w][threadIdx.x]); }
         sbox_lo[(size_t)threadIdx.x * n_super + g] = lo;
